@@ -1,0 +1,164 @@
+/*
+ * moe_a2a.h -- C ABI of the MI355X (gfx950) MoE all-to-all dispatch/combine library.
+ *
+ * One GPU holds the whole emulated world: the W destination ranks are partitions of
+ * one compact, expert-major buffer.  A routed row ("entry") is the triple
+ * (source rank, token, k); entries are numbered i = t*K + k over the tokens of all
+ * source ranks concatenated in rank order.  Entry i lives at row
+ *
+ *     slot_of_entry[i] = offsets[e_i] + #{ j < i : e_j == e_i }
+ *
+ * of disp_x[R,H], R = T*K, which is slot (owner rank e/E_l, local expert e%E_l,
+ * position j) of the reference's padded [E_l, max_recv, H] buffers
+ * (all2all/reference.py:123-146).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer into caller-owned memory unless marked host;
+ *   - the library allocates nothing, never synchronises and keeps no mutable state
+ *     besides the opt-in launch timer at the end of this file; every launch goes to
+ *     the stream passed in, so a call sequence can be captured into a hipGraph;
+ *   - return value: 0 success, < 0 argument error found on the host before any
+ *     launch (MOE_A2A_E_*), > 0 a hipError_t reported by the launch.
+ */
+#ifndef MOE_A2A_H_
+#define MOE_A2A_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_A2A_ABI_VERSION 1
+
+/* element types of activations */
+#define MOE_A2A_F16 0
+#define MOE_A2A_BF16 1
+
+/* expert stub flavours */
+#define MOE_A2A_STUB_OWNER_RANK 0      /* y = x * (1 + e / E_l)   all2all/reference.py:262 */
+#define MOE_A2A_STUB_EXPERT_FRACTION 1 /* y = x * f32((1 + e) / E)                          */
+
+/* combine arithmetic */
+#define MOE_A2A_COMBINE_STRICT 0 /* ascending slot order, round to out type after every add */
+#define MOE_A2A_COMBINE_F32 1    /* k order, f32 accumulator, one final rounding            */
+
+/* limits */
+#define MOE_A2A_MAX_EXPERTS 1024
+#define MOE_A2A_MAX_TOPK 32
+#define MOE_A2A_MAX_WORLD 256
+#define MOE_A2A_META_DIM 5
+#define MOE_A2A_FP8_BLOCK 128
+
+/* argument errors */
+#define MOE_A2A_E_NULL (-1)      /* a required pointer is NULL                       */
+#define MOE_A2A_E_SHAPE (-2)     /* T, K, E, W or H out of range / not divisible      */
+#define MOE_A2A_E_DTYPE (-3)     /* unknown element type, stub kind or combine mode   */
+#define MOE_A2A_E_WORKSPACE (-4) /* workspace missing or smaller than workspace_bytes */
+#define MOE_A2A_E_ALIGN (-5)     /* a row buffer is not 16-byte aligned               */
+#define MOE_A2A_E_STATE (-6)     /* launch timer used out of order                    */
+
+typedef void* moe_a2a_stream_t; /* hipStream_t */
+
+int moe_a2a_abi_version(void);
+
+/* Text for any value the functions below return (host pointer, static storage). */
+const char* moe_a2a_strerror(int code);
+
+/* Bytes of scratch moe_a2a_route needs for T tokens, top-K, E experts. */
+size_t moe_a2a_workspace_bytes(int T, int K, int E);
+
+/*
+ * Routing: histogram + exclusive prefix sum + stable permutation.
+ * Replaces all2all/reference.py:72-91 (bucketing, counts), :100-105 (meta rows) and
+ * :123-146 (arrival-order slotting per local expert).
+ *
+ *   indices[T,K]         expert id of every entry, 0 <= e < E
+ *   rank_start[W+1]      first token of each source rank in the concatenated world, or
+ *                        NULL: then all T tokens belong to source rank `src_rank`
+ *   counts[E]            rows per expert            (= expert_num_tokens of every rank)
+ *   offsets[E+1]         exclusive prefix sum of counts; offsets[E] = R
+ *   slot_of_entry[R]     entry -> row of the compact layout
+ *   src_of_slot[R]       row -> entry (inverse permutation)
+ *   meta[R,5]            per row: [e, source rank, token within its rank, k, 0]
+ *                        (all2all/reference.py:85)
+ *   status               optional int32[1]: set to 1 if an expert id was out of range
+ *                        (such ids are clamped into [0,E) so no access goes out of bounds)
+ */
+int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
+                  int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
+                  int32_t* status, void* workspace, size_t workspace_bytes, moe_a2a_stream_t stream);
+
+/*
+ * Dispatch: disp_x[slot_of_entry[t*K+k], :] = x[t, :] for every k.  Each token row is read
+ * once and stored K times.  Pure copy of 16-bit elements (H % 8 == 0).
+ * Replaces all2all/reference.py:93-112 (send-buffer gather + exchange) and :144.
+ */
+int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, int T, int K, int H,
+                     moe_a2a_stream_t stream);
+
+/*
+ * Routing and dispatch in ONE launch for small worlds (R = T*K <= moe_a2a_fused_max_rows()):
+ * every workgroup derives the slots of its own token from the routing table, so no
+ * routing kernel has to finish first.  Outputs as moe_a2a_route + moe_a2a_dispatch.
+ */
+int moe_a2a_fused_max_rows(void);
+int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
+                           int K, int E, int W, int H, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
+                           int32_t* src_of_slot, int32_t* meta, int32_t* status, void* disp_x,
+                           moe_a2a_stream_t stream);
+
+/*
+ * fp8 dispatch: quantise each token row once to e4m3fn with one f32 scale per 128 columns
+ * (scale = amax/448, 1 if amax == 0; q = rne_e4m3(x / scale)), then store row and scales at
+ * the K slots.  x is MOE_A2A_F16 or MOE_A2A_BF16, H % 128 == 0.  The reference has no fp8
+ * path; the arithmetic is the one stated here.
+ *   disp_q[R,H] uint8, disp_scale[R,H/128] f32
+ */
+int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry, uint8_t* disp_q,
+                         float* disp_scale, int T, int K, int H, moe_a2a_stream_t stream);
+
+/*
+ * Expert stub (all2all/reference.py:262): y[row,:] = round_out(f32(round_out(x[row,:])) * s(e)),
+ * e = meta[row,0].  With disp_scale != NULL the input is fp8: y = round_out((f32(q)*scale) * s(e)).
+ */
+int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta, int in_type, int out_type,
+                 int stub_kind, int E, int W, void* y, int R, int H, moe_a2a_stream_t stream);
+
+/*
+ * Combine: out[t,:] = sum_k weights[t,k] * expert_y[slot_of_entry[t*K+k], :]
+ * (all2all/reference.py:163-232 without the regroup/exchange).  STRICT reproduces the
+ * reference's order (ascending slot) and its rounding to the output type after every add;
+ * F32 keeps an f32 accumulator in k order.  Multiply and add are never contracted.
+ * Rows of out that belong to no token are not touched.
+ */
+int moe_a2a_combine(const void* expert_y, const float* weights, const int32_t* slot_of_entry, int mode,
+                    int elem_type, void* out, int T, int K, int H, moe_a2a_stream_t stream);
+
+/*
+ * Combine with the expert stub folded in: reads the dispatched rows directly and applies
+ * s(e) with the stub's rounding before the weighted sum -- identical results to
+ * moe_a2a_stub followed by moe_a2a_combine, without the R*H round trip through memory.
+ */
+int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_t* indices,
+                         const float* weights, const int32_t* slot_of_entry, int mode, int in_type, int out_type,
+                         int stub_kind, int E, int W, void* out, int T, int K, int H, moe_a2a_stream_t stream);
+
+/*
+ * Launch timer (opt-in, process-wide, single caller thread).  Between begin and end every
+ * kernel the library launches carries a pair of HIP events bound to that dispatch, so the
+ * reported time is the kernel's own begin-to-end duration on the GPU.
+ *   begin(capacity)  allocate `capacity` event pairs and start recording
+ *   end(ids, us, n)  wait for the recorded launches, write up to n (kernel id, microseconds)
+ *                    pairs to HOST arrays, release the events; returns the number written
+ *   kernel_name(id)  host string for a kernel id
+ */
+int moe_a2a_timer_begin(int capacity);
+int moe_a2a_timer_end(int* kernel_ids, float* microseconds, int n);
+const char* moe_a2a_kernel_name(int kernel_id);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_A2A_H_ */

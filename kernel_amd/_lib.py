@@ -1,0 +1,72 @@
+"""ctypes binding of ``libmoe_a2a.so`` (declared in include/moe_a2a.h).
+
+There is no fallback: if the library is missing, ``load()`` raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmoe_a2a.so")
+
+ABI_VERSION = 1
+F16, BF16 = 0, 1
+
+_i32p = C.c_void_p  # device pointers travel as plain addresses
+_vp = C.c_void_p
+_int = C.c_int
+
+# name -> (restype, argtypes); mirrors include/moe_a2a.h one to one
+PROTOTYPES = {
+    "moe_a2a_abi_version": (_int, []),
+    "moe_a2a_strerror": (C.c_char_p, [_int]),
+    "moe_a2a_workspace_bytes": (C.c_size_t, [_int, _int, _int]),
+    "moe_a2a_route": (_int, [_i32p, _i32p, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p, _i32p, _i32p, _i32p,
+                             _vp, C.c_size_t, _vp]),
+    "moe_a2a_dispatch": (_int, [_vp, _i32p, _vp, _int, _int, _int, _vp]),
+    "moe_a2a_fused_max_rows": (_int, []),
+    "moe_a2a_route_dispatch": (_int, [_vp, _i32p, _i32p, _int, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p,
+                                      _i32p, _i32p, _i32p, _vp, _vp]),
+    "moe_a2a_dispatch_fp8": (_int, [_vp, _int, _i32p, _vp, _vp, _int, _int, _int, _vp]),
+    "moe_a2a_stub": (_int, [_vp, _vp, _i32p, _int, _int, _int, _int, _int, _vp, _int, _int, _vp]),
+    "moe_a2a_combine": (_int, [_vp, _vp, _i32p, _int, _int, _vp, _int, _int, _int, _vp]),
+    "moe_a2a_stub_combine": (_int, [_vp, _vp, _i32p, _vp, _i32p, _int, _int, _int, _int, _int, _int, _vp, _int, _int,
+                                    _int, _vp]),
+    "moe_a2a_timer_begin": (_int, [_int]),
+    "moe_a2a_timer_end": (_int, [C.POINTER(C.c_int), C.POINTER(C.c_float), _int]),
+    "moe_a2a_kernel_name": (C.c_char_p, [_int]),
+}
+
+_lib = None
+
+
+class MoeA2AError(RuntimeError):
+    def __init__(self, code: int, where: str):
+        self.code = code
+        msg = load().moe_a2a_strerror(code)
+        super().__init__(f"{where}: {msg.decode() if msg else 'error'} (code {code})")
+
+
+def load() -> C.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m kernel_amd.build` (there is no fallback path)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    got = lib.moe_a2a_abi_version()
+    if got != ABI_VERSION:
+        raise RuntimeError(f"libmoe_a2a.so has ABI {got}, binding expects {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def check(code: int, where: str) -> None:
+    if code != 0:
+        raise MoeA2AError(code, where)

@@ -1,0 +1,270 @@
+"""Host side of the MoE all-to-all: same roles as the reference's ``PyTorchAllToAll``
+(all2all/reference.py:55-234), every step a HIP kernel behind the C ABI.
+
+``HipAllToAll(cfg, rank, world_size)`` offers ``dispatch`` -> ``expert_stub`` ->
+``combine``.  Differences from the reference that a caller sees:
+
+* one GPU holds every destination rank, so ``dispatch`` returns the rows of ALL
+  ``num_experts`` experts in one compact expert-major buffer (``Dispatched``) instead of
+  the calling rank's padded ``[E_l, max_recv, H]`` slice; ``Dispatched.padded(owner)``
+  rebuilds the reference's triple for one owner rank;
+* there is no process group: the three exchanges per phase are gone;
+* ``combine`` writes ``out[:T]`` (it does not add into what ``out`` held before).
+
+torch is used for device memory and the current stream only.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from .contract import (COMBINE_F32, COMBINE_STRICT, FP8_BLOCK, META_DIM, STUB_EXPERT_FRACTION, STUB_OWNER_RANK,
+                       MoEConfig)
+
+_ELEM = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+
+
+def _elem(dtype: torch.dtype) -> int:
+    try:
+        return _ELEM[dtype]
+    except KeyError:
+        raise TypeError(f"activations must be float16 or bfloat16, got {dtype}") from None
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU: the HIP library is the only implementation")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+@dataclasses.dataclass
+class Dispatched:
+    """Result of ``dispatch``: the compact expert-major layout of the whole world."""
+
+    cfg: MoEConfig
+    world_size: int
+    num_tokens: int  # T, tokens of all source ranks
+    counts: torch.Tensor  # [E]   int32 rows per expert (= expert_num_tokens of every rank, concatenated)
+    offsets: torch.Tensor  # [E+1] int32 first row of each expert
+    slot_of_entry: torch.Tensor  # [R] int32
+    src_of_slot: torch.Tensor  # [R] int32
+    meta: torch.Tensor  # [R,5] int32: e, source rank, token in rank, k, 0
+    disp_x: torch.Tensor  # [R,H] in_dtype, or uint8 e4m3fn bits for fp8 dispatch
+    disp_scale: Optional[torch.Tensor] = None  # [R,H/128] f32 (fp8 only)
+    status: Optional[torch.Tensor] = None  # [1] int32, 1 if an expert id was out of range
+
+    @property
+    def num_rows(self) -> int:
+        return self.slot_of_entry.numel()
+
+    def padded(self, owner_rank: int, max_recv: Optional[int] = None):
+        """``(expert_num_tokens, expert_x, expert_meta)`` of one owner rank in the reference's
+        padded shape (all2all/reference.py:123-148); rows past the count are zero."""
+        cfg, W = self.cfg, self.world_size
+        E_l = cfg.num_experts // W
+        max_recv = max_recv if max_recv is not None else cfg.max_num_tokens * W
+        lo, hi = owner_rank * E_l, (owner_rank + 1) * E_l
+        num = self.counts[lo:hi].clone()
+        off = self.offsets[lo:hi + 1].tolist()
+        ex = torch.zeros(E_l, max_recv, self.disp_x.shape[1], dtype=self.disp_x.dtype, device=self.disp_x.device)
+        em = torch.zeros(E_l, max_recv, META_DIM, dtype=torch.int32, device=self.meta.device)
+        for le in range(E_l):
+            n = off[le + 1] - off[le]
+            if n > max_recv:
+                raise ValueError(f"expert {lo + le} holds {n} rows, more than max_recv={max_recv}")
+            ex[le, :n] = self.disp_x[off[le]:off[le + 1]]
+            em[le, :n] = self.meta[off[le]:off[le + 1]]
+        return num, ex, em
+
+
+class HipAllToAll:
+    """MoE dispatch / expert stub / combine on one MI355X."""
+
+    META_DIM = META_DIM
+
+    def __init__(self, cfg: MoEConfig, rank: int, world_size: int, stub_kind: int = STUB_OWNER_RANK,
+                 combine_mode: int = COMBINE_STRICT, fp8_dispatch: bool = False, fuse_route: bool = True,
+                 fuse_stub: bool = False):
+        if cfg.num_experts % world_size:
+            raise ValueError("num_experts must be a multiple of world_size")
+        self.cfg = cfg
+        self.rank = rank
+        self.world_size = world_size
+        self.num_local_experts = cfg.num_experts // world_size
+        self.max_recv = cfg.max_num_tokens * world_size
+        self.stub_kind = stub_kind
+        self.combine_mode = combine_mode
+        self.fp8_dispatch = fp8_dispatch
+        self.fuse_route = fuse_route
+        self.fuse_stub = fuse_stub
+        self.lib = _lib.load()
+        self._fused_max_rows = self.lib.moe_a2a_fused_max_rows()
+        self._bufs = {}
+
+    # ---- buffers ---------------------------------------------------------------------
+    def _buffers(self, T: int, device) -> dict:
+        """Device buffers for T tokens, kept between calls (a call overwrites all of them)."""
+        key = (T, str(device))
+        b = self._bufs.get(key)
+        if b is not None:
+            return b
+        cfg = self.cfg
+        K, H, E = cfg.experts_per_token, cfg.hidden_dim, cfg.num_experts
+        R = T * K
+        i32 = dict(dtype=torch.int32, device=device)
+        b = dict(
+            counts=torch.empty(E, **i32),
+            offsets=torch.empty(E + 1, **i32),
+            slot_of_entry=torch.empty(R, **i32),
+            src_of_slot=torch.empty(R, **i32),
+            meta=torch.empty(R, META_DIM, **i32),
+            status=torch.zeros(1, **i32),
+            workspace=torch.empty(max(self.lib.moe_a2a_workspace_bytes(T, K, E), 256), dtype=torch.uint8,
+                                  device=device),
+            expert_y=torch.empty(R, H, dtype=cfg.out_dtype, device=device),
+            out=torch.empty(T, H, dtype=cfg.out_dtype, device=device),
+        )
+        if self.fp8_dispatch:
+            b["disp_x"] = torch.empty(R, H, dtype=torch.uint8, device=device)
+            b["disp_scale"] = torch.empty(R, H // FP8_BLOCK, dtype=torch.float32, device=device)
+        else:
+            b["disp_x"] = torch.empty(R, H, dtype=cfg.in_dtype, device=device)
+            b["disp_scale"] = None
+        self._bufs[key] = b
+        return b
+
+    def release_buffers(self) -> None:
+        self._bufs.clear()
+
+    # ---- dispatch --------------------------------------------------------------------
+    def dispatch(self, dp_x: torch.Tensor, indices: torch.Tensor,
+                 rank_start: Optional[torch.Tensor] = None) -> Dispatched:
+        """all2all/reference.py:68-148.
+
+        ``dp_x[T,H]`` and ``indices[T,K]`` are the tokens of this rank, or of the whole world
+        concatenated in rank order when ``rank_start[W+1]`` (int32, on the GPU) is given.
+        """
+        cfg = self.cfg
+        _require_gpu(dp_x, "dp_x")
+        _require_gpu(indices, "indices")
+        if indices.dtype != torch.int32:
+            raise TypeError("indices must be int32")
+        T, H = dp_x.shape
+        K, E, W = cfg.experts_per_token, cfg.num_experts, self.world_size
+        if H != cfg.hidden_dim or tuple(indices.shape) != (T, K) or dp_x.dtype != cfg.in_dtype:
+            raise ValueError("dp_x / indices do not match the MoEConfig")
+        if rank_start is not None:
+            _require_gpu(rank_start, "rank_start")
+            if rank_start.dtype != torch.int32 or rank_start.numel() != W + 1:
+                raise ValueError("rank_start must be int32[world_size + 1]")
+        b = self._buffers(T, dp_x.device)
+        lib, st = self.lib, _stream()
+        route_out = (_ptr(b["counts"]), _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]),
+                     _ptr(b["meta"]), _ptr(b["status"]))
+        if self.fuse_route and not self.fp8_dispatch and 0 < T * K <= self._fused_max_rows:
+            _lib.check(lib.moe_a2a_route_dispatch(_ptr(dp_x), _ptr(indices), _ptr(rank_start), self.rank, T, K, E, W,
+                                                  H, *route_out, _ptr(b["disp_x"]), st), "moe_a2a_route_dispatch")
+        else:
+            _lib.check(lib.moe_a2a_route(_ptr(indices), _ptr(rank_start), self.rank, T, K, E, W, *route_out,
+                                         _ptr(b["workspace"]), b["workspace"].numel(), st), "moe_a2a_route")
+            if self.fp8_dispatch:
+                _lib.check(lib.moe_a2a_dispatch_fp8(_ptr(dp_x), _elem(cfg.in_dtype), _ptr(b["slot_of_entry"]),
+                                                    _ptr(b["disp_x"]), _ptr(b["disp_scale"]), T, K, H, st),
+                           "moe_a2a_dispatch_fp8")
+            else:
+                _lib.check(lib.moe_a2a_dispatch(_ptr(dp_x), _ptr(b["slot_of_entry"]), _ptr(b["disp_x"]), T, K, H, st),
+                           "moe_a2a_dispatch")
+        return Dispatched(cfg, W, T, b["counts"], b["offsets"], b["slot_of_entry"], b["src_of_slot"], b["meta"],
+                          b["disp_x"], b["disp_scale"], b["status"])
+
+    # ---- expert stub -----------------------------------------------------------------
+    def expert_stub(self, d: Dispatched) -> torch.Tensor:
+        """all2all/reference.py:262 on the compact rows -> ``expert_y[R,H]`` out_dtype."""
+        cfg = self.cfg
+        R, H = d.disp_x.shape
+        y = self._buffers(d.num_tokens, d.disp_x.device)["expert_y"]
+        in_type = _lib.BF16 if d.disp_scale is not None else _elem(d.disp_x.dtype)
+        _lib.check(self.lib.moe_a2a_stub(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(d.meta), in_type,
+                                         _elem(cfg.out_dtype), self.stub_kind, cfg.num_experts, self.world_size,
+                                         _ptr(y), R, H, _stream()), "moe_a2a_stub")
+        return y
+
+    # ---- combine ---------------------------------------------------------------------
+    def combine(self, out_tokens: Optional[torch.Tensor], weights: torch.Tensor, d: Dispatched,
+                expert_y: torch.Tensor) -> torch.Tensor:
+        """all2all/reference.py:151-234: weighted sum of each token's K expert rows into
+        ``out_tokens[:T]`` (allocated here when None)."""
+        cfg = self.cfg
+        T, K, H = d.num_tokens, cfg.experts_per_token, cfg.hidden_dim
+        _require_gpu(weights, "weights")
+        _require_gpu(expert_y, "expert_y")
+        if weights.dtype != torch.float32 or tuple(weights.shape) != (T, K):
+            raise ValueError("weights must be float32[T,K]")
+        if expert_y.dtype != cfg.out_dtype or tuple(expert_y.shape) != (T * K, H):
+            raise ValueError("expert_y must be out_dtype[T*K,H]")
+        if out_tokens is None:
+            out_tokens = self._buffers(T, expert_y.device)["out"]
+        else:
+            _require_gpu(out_tokens, "out_tokens")
+            if out_tokens.dtype != cfg.out_dtype or out_tokens.shape[0] < T or out_tokens.shape[1] != H:
+                raise ValueError("out_tokens must be out_dtype[>=T,H]")
+        _lib.check(self.lib.moe_a2a_combine(_ptr(expert_y), _ptr(weights), _ptr(d.slot_of_entry), self.combine_mode,
+                                            _elem(cfg.out_dtype), _ptr(out_tokens), T, K, H, _stream()),
+                   "moe_a2a_combine")
+        return out_tokens
+
+    def stub_combine(self, out_tokens: Optional[torch.Tensor], weights: torch.Tensor, indices: torch.Tensor,
+                     d: Dispatched) -> torch.Tensor:
+        """Expert stub folded into the combine (same results, no ``expert_y`` buffer)."""
+        cfg = self.cfg
+        T, K, H = d.num_tokens, cfg.experts_per_token, cfg.hidden_dim
+        _require_gpu(weights, "weights")
+        _require_gpu(indices, "indices")
+        if out_tokens is None:
+            out_tokens = self._buffers(T, weights.device)["out"]
+        in_type = _lib.BF16 if d.disp_scale is not None else _elem(d.disp_x.dtype)
+        _lib.check(self.lib.moe_a2a_stub_combine(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(indices), _ptr(weights),
+                                                 _ptr(d.slot_of_entry), self.combine_mode, in_type,
+                                                 _elem(cfg.out_dtype), self.stub_kind, cfg.num_experts,
+                                                 self.world_size, _ptr(out_tokens), T, K, H, _stream()),
+                   "moe_a2a_stub_combine")
+        return out_tokens
+
+    # ---- whole path ------------------------------------------------------------------
+    def forward(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
+                rank_start: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """dispatch -> stub -> combine; returns ``y[T,H]`` (a buffer the next call reuses)."""
+        if x.shape[0] == 0:
+            return torch.empty(0, self.cfg.hidden_dim, dtype=self.cfg.out_dtype, device=x.device)
+        d = self.dispatch(x, indices, rank_start)
+        if self.fuse_stub:
+            return self.stub_combine(None, weights, indices, d)
+        return self.combine(None, weights, d, self.expert_stub(d))
+
+
+def concat_world(world: Sequence, device=None):
+    """Concatenate per-rank records in rank order -> x, indices, weights, rank_start (int32)."""
+    x = torch.cat([rd.x for rd in world], 0)
+    idx = torch.cat([rd.indices for rd in world], 0)
+    w = torch.cat([rd.weights for rd in world], 0)
+    starts = [0]
+    for rd in world:
+        starts.append(starts[-1] + int(rd.num_tokens))
+    rs = torch.tensor(starts, dtype=torch.int32)
+    if device is not None:
+        x, idx, w, rs = x.to(device), idx.to(device), w.to(device), rs.to(device)
+    else:
+        rs = rs.to(x.device)
+    return x.contiguous(), idx.contiguous(), w.contiguous(), rs

@@ -1,0 +1,39 @@
+"""``custom_kernel(data)`` -- the entry point a caller of the reference imports from its
+``submission`` module (eval.py:159-180; shape of the call: submission.py:192-219).
+
+``data = (cfg, rank_data, rank, world_size)``; returns ``y[:num_tokens]`` with dtype
+``cfg.out_dtype`` on the device of ``rank_data.x``.  The destination ranks are partitions
+of one buffer on that GPU, so no process group is needed and every emulated rank may
+call this from one process.  The expert stand-in is the reference's ``x * (1 + owner)``.
+"""
+from __future__ import annotations
+
+import torch
+
+from .all2all import HipAllToAll
+from .contract import COMBINE_STRICT, STUB_OWNER_RANK
+
+_instances = {}
+
+
+def _instance(cfg, rank: int, world_size: int, device, stub_kind: int, combine_mode: int) -> HipAllToAll:
+    key = (cfg.num_experts, cfg.experts_per_token, cfg.hidden_dim, cfg.in_dtype, cfg.out_dtype, rank, world_size,
+           str(device), stub_kind, combine_mode)
+    ata = _instances.get(key)
+    if ata is None:
+        if len(_instances) > 64:
+            _instances.clear()
+        ata = _instances[key] = HipAllToAll(cfg, rank, world_size, stub_kind=stub_kind, combine_mode=combine_mode)
+    return ata
+
+
+def custom_kernel(data, stub_kind: int = STUB_OWNER_RANK, combine_mode: int = COMBINE_STRICT) -> torch.Tensor:
+    cfg, rank_data, rank, world_size = data
+    x = rank_data.x
+    if not x.is_cuda:
+        raise RuntimeError("custom_kernel needs its inputs on the GPU: there is no CPU implementation")
+    ata = _instance(cfg, rank, world_size, x.device, stub_kind, combine_mode)
+    with torch.cuda.device(x.device):
+        y = ata.forward(x.contiguous(), rank_data.indices.contiguous(), rank_data.weights.contiguous())
+    # the caller owns its result (eval.py deletes it after each run): hand out a copy of the reused buffer
+    return y[: rank_data.num_tokens].clone()

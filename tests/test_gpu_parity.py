@@ -1,0 +1,144 @@
+"""HIP path against the CPU oracle, through the C ABI, on seeded inputs.  Needs a GPU.
+
+Bar: counts, offsets, permutations, meta, dispatched rows, stub rows and the combine output
+are compared BIT FOR BIT (both combine modes follow a stated operation order, so they are
+exact too); fp8 rows are compared bit for bit against torch's e4m3fn cast.
+"""
+import pytest
+import torch
+
+from golden_io import GOLDEN_CASES, bits, golden_compact, load_golden
+from kernel_amd import contract as C
+from kernel_amd.all2all import HipAllToAll, concat_world
+from oracle import all2all_vec as V
+
+pytestmark = pytest.mark.gpu
+
+
+def run_hip(cfg, world, dev, stub_kind, combine_mode=0, fp8=False, fuse_route=True, rank=0):
+    W = len(world)
+    x, idx, w, rs = concat_world(world, dev)
+    ata = HipAllToAll(cfg, rank, W, stub_kind=stub_kind, combine_mode=combine_mode, fp8_dispatch=fp8,
+                      fuse_route=fuse_route)
+    d = ata.dispatch(x, idx, rs)
+    ey = ata.expert_stub(d)
+    y = ata.combine(None, w, d, ey)
+    y2 = ata.stub_combine(torch.empty_like(y), w, idx, d)
+    torch.cuda.synchronize()
+    return d, ey, y, y2
+
+
+def assert_same(name, got, want):
+    got = got.cpu()
+    assert got.shape == want.shape, f"{name}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    assert got.dtype == want.dtype, f"{name}: dtype {got.dtype} != {want.dtype}"
+    g, w = bits(got), bits(want)
+    if not torch.equal(g, w):
+        bad = (g != w).nonzero()
+        raise AssertionError(f"{name}: {bad.shape[0]} mismatches, first at {bad[0].tolist()}: "
+                             f"{got[tuple(bad[0])]} != {want[tuple(bad[0])]}")
+
+
+def compare(cfg, world, dev, stub_kind, combine_mode=0, fp8=False, fuse_route=True):
+    o = V.run_world(cfg, world, stub_kind=stub_kind, fp8=fp8, combine_mode=combine_mode)
+    d, ey, y, y2 = run_hip(cfg, world, dev, stub_kind, combine_mode, fp8, fuse_route)
+    assert int(d.status.item()) == 0
+    assert_same("counts", d.counts, o["counts"])
+    assert_same("offsets", d.offsets, o["offsets"])
+    assert_same("slot_of_entry", d.slot_of_entry, o["slot_of_entry"])
+    assert_same("src_of_slot", d.src_of_slot, o["src_of_slot"])
+    assert_same("meta", d.meta, o["meta"])
+    assert_same("disp_x", d.disp_x, o["disp_x"])
+    if fp8:
+        assert_same("disp_scale", d.disp_scale, o["disp_scale"])
+    assert_same("expert_y", ey, o["expert_y"])
+    assert_same("y", y, o["y"])
+    assert_same("y (stub folded into combine)", y2, o["y"])
+    return o, d
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+@pytest.mark.parametrize("fuse_route", [True, False])
+def test_reference_vectors(gpu_device, name, fuse_route):
+    """Against the outputs the reference's own PyTorchAllToAll wrote (tests/golden/)."""
+    cfg, world, expected = load_golden(name)
+    g = golden_compact(cfg, expected)
+    d, ey, y, y2 = run_hip(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=fuse_route)
+    assert_same("counts", d.counts, g["counts"])
+    assert_same("meta", d.meta, g["meta"])
+    assert_same("disp_x", d.disp_x, g["disp_x"])
+    assert_same("expert_y", ey, g["expert_y"])
+    assert_same("y", y, g["y"])
+    assert_same("y2", y2, g["y"])
+    # the reference's own return value of dispatch for every owner rank
+    for r, exp in enumerate(expected):
+        num, ex, em = d.padded(r)
+        assert_same("expert_num_tokens", num, exp.expert_num_tokens)
+        rows = torch.cat([ex[le, : int(num[le])] for le in range(num.numel())], 0)
+        assert_same("expert_x", rows, exp.expert_x)
+
+
+@pytest.mark.parametrize("spec", C.REFERENCE_TESTS, ids=lambda s: f"E{s['num_experts']}K{s['experts_per_token']}"
+                                                                     f"H{s['hidden_dim']}T{s['max_num_tokens']}")
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+def test_reference_specs_whole_world(gpu_device, spec, dtype):
+    """The reference's 9 test specs (all2all/task.yml:59-68), all 8 ranks resident at once."""
+    cfg, world = C.generate_world(**spec, dtype=dtype)
+    for fuse in (True, False):
+        compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=fuse)
+
+
+@pytest.mark.parametrize("name,scale", [("tiny", 1.0), ("dsv3_rank", 1.0), ("skew_world", 1.0)])
+@pytest.mark.parametrize("mode", [C.COMBINE_STRICT, C.COMBINE_F32], ids=["strict", "f32"])
+def test_named_workloads(gpu_device, name, scale, mode):
+    wl = C.generate_workload(name, tokens_scale=scale)
+    for fuse in (True, False):
+        o, d = compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, combine_mode=mode, fuse_route=fuse)
+    if name == "skew_world":
+        assert int(o["counts"].max()) <= wl.total_tokens  # one row per token and expert at most
+
+
+def test_multi_workgroup_routing(gpu_device):
+    """R = 40960 > one-workgroup limit: histogram / scan / rank kernels, 8 source ranks."""
+    wl = C.generate_workload("prefill_graph", tokens_scale=10240 / 16384)
+    cfg = wl.cfg
+    # spread the tokens over 8 uneven source ranks
+    x, idx, w = wl.world[0].x, wl.world[0].indices, wl.world[0].weights
+    cuts = [0, 7, 7, 3000, 3001, 6000, 9000, 10239, 10240]
+    world = [C.RankData(cuts[i + 1] - cuts[i], idx[cuts[i]:cuts[i + 1]], w[cuts[i]:cuts[i + 1]],
+                        x[cuts[i]:cuts[i + 1]]) for i in range(8)]
+    compare(cfg, world, gpu_device, C.STUB_EXPERT_FRACTION)
+
+
+def test_fp8_dispatch(gpu_device):
+    wl = C.generate_workload("fp8_dispatch", tokens_scale=512 / 4096)
+    compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, fp8=True)
+    compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, fp8=True, combine_mode=C.COMBINE_F32)
+
+
+def test_duplicate_experts_and_ragged_world(gpu_device):
+    """A token may name the same expert twice; ranks may be empty; H not a multiple of 256 lanes."""
+    g = torch.Generator().manual_seed(5)
+    cfg = C.MoEConfig(16, 4, 2880, 9, torch.bfloat16, torch.bfloat16)
+    world = []
+    for n in [3, 0, 8, 1]:
+        world.append(C.RankData(n, torch.randint(0, 16, (n, 4), generator=g).to(torch.int32),
+                                torch.rand(n, 4, generator=g), torch.randn(n, 2880, generator=g).to(torch.bfloat16)))
+    for fuse in (True, False):
+        compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=fuse)
+
+
+def test_custom_kernel_contract(gpu_device):
+    """custom_kernel(data) per rank == oracle ref_kernel, checked with the reference's tolerance."""
+    from kernel_amd.submission import custom_kernel
+    from oracle.checker import check_implementation, ref_kernel
+
+    spec = dict(C.REFERENCE_TESTS[5])
+    W = spec.pop("world_size")
+    for rank in range(W):
+        data = C.generate_input(**spec, rank=rank, world_size=W, device=gpu_device)
+        out = custom_kernel(data)
+        assert out.dtype == data[0].out_dtype and out.shape == (data[1].num_tokens, data[0].hidden_dim)
+        ok, msg = check_implementation(data, out)
+        assert ok, msg
+        assert torch.equal(bits(out.cpu()), bits(ref_kernel(data).cpu()))
