@@ -1,0 +1,246 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE dispatch -> expert stub -> combine path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload dsv3_rank]
+
+A step is one pass of the path over one resident batch: routing + dispatch, expert stub,
+combine (three launches at the default workload), replayed from a hipGraph.  Inputs are in
+HBM before the timed region starts.  Prints ONE JSON line:
+
+  value        achieved GB/s of dispatch+combine: algorithmic bytes (read x once, write R
+               rows; read R rows, write T rows) / summed GPU durations of the routing,
+               dispatch and combine kernels of a step.  Kernel durations come from HIP
+               events bound to each launch, on the stream the kernels run on.
+  ms_per_step  wall time of a whole step (including the stub launch), events around K steps.
+  roofline     the slower of the dispatch / combine kernels against the 8 TB/s HBM peak.
+  cpu_baseline the CPU oracle (a port of the reference's torch path) timed on the host
+               cores for the same workload, and used to check the GPU result.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "dispatch+combine µs and achieved HBM GB/s (% of peak), 256E/top8/h7168 bf16"
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--workload", default="dsv3_rank")
+    p.add_argument("--combine", choices=["strict", "f32"], default="strict")
+    p.add_argument("--no-graph", action="store_true", help="launch eagerly from Python instead of a hipGraph")
+    p.add_argument("--no-fuse-route", action="store_true", help="separate routing kernel even for small worlds")
+    p.add_argument("--fuse-stub", action="store_true", help="fold the expert stub into the combine")
+    p.add_argument("--bf16-dispatch", action="store_true", help="fp8 workload with a 16-bit dispatch")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--no-cold", action="store_true", help="skip the cold-cache leg")
+    p.add_argument("--cpu-seconds", type=float, default=12.0)
+    return p.parse_args()
+
+
+def kernel_times(lib, run, steps, torch):
+    """Per-kernel GPU durations (µs) of `steps` eager passes, from the library's launch timer."""
+    cap = steps * 8
+    rc = lib.moe_a2a_timer_begin(cap)
+    if rc != 0:
+        raise RuntimeError(f"moe_a2a_timer_begin: {lib.moe_a2a_strerror(rc).decode()}")
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    ids = (ctypes.c_int * cap)()
+    us = (ctypes.c_float * cap)()
+    n = lib.moe_a2a_timer_end(ids, us, cap)
+    per = {}
+    for i in range(n):
+        per.setdefault(lib.moe_a2a_kernel_name(ids[i]).decode(), []).append(float(us[i]))
+    return per
+
+
+def summarise(per):
+    return {k: dict(mean_us=round(statistics.fmean(v), 3), min_us=round(min(v), 3),
+                    median_us=round(statistics.median(v), 3), launches=len(v)) for k, v in per.items()}
+
+
+ROUTE_KERNELS = ("route_single", "route_hist", "route_scan", "route_rank")
+DISPATCH_KERNELS = ("dispatch_rows", "route_dispatch", "dispatch_fp8")
+COMBINE_KERNELS = ("combine_rows", "stub_combine")
+STUB_KERNELS = ("stub_rows", "stub_fp8")
+
+
+def per_step(per, names, steps):
+    return sum(sum(per.get(n, [])) for n in names) / steps
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: the emulated destination ranks are partitions of one HBM buffer and "
+              f"there is no cross-GPU path in this build (got --gpus {args.gpus}).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from kernel_amd import _lib, contract
+    from kernel_amd.all2all import HipAllToAll, concat_world
+
+    lib = _lib.load()
+    if not torch.cuda.is_available():
+        raise RuntimeError("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    wl = contract.generate_workload(args.workload)
+    cfg, W = wl.cfg, wl.world_size
+    T, K, H, E = wl.total_tokens, cfg.experts_per_token, cfg.hidden_dim, cfg.num_experts
+    fp8 = wl.fp8_dispatch and not args.bf16_dispatch
+    mode = contract.COMBINE_STRICT if args.combine == "strict" else contract.COMBINE_F32
+    ata = HipAllToAll(cfg, 0, W, stub_kind=wl.stub_kind, combine_mode=mode, fp8_dispatch=fp8,
+                      fuse_route=not args.no_fuse_route, fuse_stub=args.fuse_stub)
+    x, idx, w, rs = concat_world(wl.world, dev)
+
+    def step():
+        return ata.forward(x, idx, w, rs)
+
+    y = step()
+    torch.cuda.synchronize()
+    run = step
+    use_graph = not args.no_graph
+    if use_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = step()
+        run = graph.replay
+
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+
+    # per-kernel durations: eager launches, each carrying its own pair of HIP events
+    for _ in range(3):
+        step()
+    per = kernel_times(lib, step, args.steps, torch)
+    t_route = per_step(per, ROUTE_KERNELS, args.steps)
+    t_disp = per_step(per, DISPATCH_KERNELS, args.steps)
+    t_comb = per_step(per, COMBINE_KERNELS, args.steps)
+    t_stub = per_step(per, STUB_KERNELS, args.steps)
+    ab = contract.algorithmic_bytes(T, K, H, 2, 2, fp8)
+    b_dc = ab["dispatch"] + ab["combine"]
+    t_dc = t_route + t_disp + t_comb
+    value = b_dc / t_dc / 1e3  # bytes/µs -> GB/s
+
+    # dominant kernel for the roofline entry
+    disp_name = next(n for n in DISPATCH_KERNELS if n in per)
+    comb_name = next(n for n in COMBINE_KERNELS if n in per)
+    cand = [(disp_name, ab["dispatch"]), (comb_name, ab["combine"])]
+    dom_name, dom_bytes = max(cand, key=lambda c: statistics.fmean(per[c[0]]))
+    dom_us = statistics.fmean(per[dom_name])
+    roofline = dict(bound="hbm", kernel=dom_name, achieved=round(dom_bytes / dom_us / 1e3, 1), peak=HBM_PEAK_GBPS,
+                    unit="GB/s", frac=round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
+                    bytes_per_launch=dom_bytes, avg_us=round(dom_us, 3), traffic=None)
+
+    out = dict(
+        metric=METRIC, value=round(value, 1), unit="GB/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
+        ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
+        dtype="fp8-e4m3 dispatch, bf16 combine" if fp8 else str(cfg.in_dtype).replace("torch.", ""),
+        data="synthetic",
+        config=dict(workload=args.workload, tokens=T, experts=E, top_k=K, hidden=H, emulated_ranks=W,
+                    routed_rows=T * K, combine=args.combine, launch="hipGraph replay" if use_graph else "eager",
+                    fused_route=bool(not args.no_fuse_route and not fp8 and T * K <= lib.moe_a2a_fused_max_rows()),
+                    fused_stub=bool(args.fuse_stub)),
+        dispatch_combine_us=round(t_dc, 3), route_us=round(t_route, 3), dispatch_us=round(t_disp, 3),
+        stub_us=round(t_stub, 3), combine_us=round(t_comb, 3),
+        pct_of_hbm_peak=round(100.0 * value / HBM_PEAK_GBPS, 2),
+        tokens_per_s=round(T / (t_dc * 1e-6), 1),
+        tokens_per_s_wall=round(T / (ms_per_step * 1e-3), 1),
+        bytes=dict(dispatch=ab["dispatch"], combine=ab["combine"], stub=ab["stub"]),
+        kernels=summarise(per),
+        roofline=roofline,
+    )
+
+    if not args.no_cold:
+        # cold caches: overwrite 1 GiB (4x the 256 MB Infinity Cache) before every step
+        flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        n_cold = min(args.steps, 30)
+
+        def cold_step():
+            flush.fill_(1)
+            step()
+
+        cold_step()
+        perc = kernel_times(lib, cold_step, n_cold, torch)
+        tc = per_step(perc, ROUTE_KERNELS + DISPATCH_KERNELS + COMBINE_KERNELS, n_cold)
+        out["cold"] = dict(dispatch_combine_us=round(tc, 3), GBps=round(b_dc / tc / 1e3, 1),
+                           pct_of_hbm_peak=round(100.0 * b_dc / tc / 1e3 / HBM_PEAK_GBPS, 2),
+                           kernels={k: v["mean_us"] for k, v in summarise(perc).items()})
+        del flush
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(wl, mode, fp8, y, b_dc, args.cpu_seconds)
+    print(json.dumps(out, ensure_ascii=False), flush=True)
+
+
+def cpu_baseline(wl, mode, fp8, y_gpu, b_dc, budget_s):
+    """The CPU oracle on the host cores: same workload, same bytes; also checks the GPU output."""
+    import torch
+
+    from oracle import all2all_vec as V  # checker and baseline only
+
+    cfg = wl.cfg
+    K = cfg.experts_per_token
+    x, idx, w, starts = V.concat_world(wl.world)
+    comb = V.combine_strict if mode == 0 else V.combine_f32
+    times = []
+    t_begin = time.perf_counter()
+    y_cpu = None
+    while True:
+        t0 = time.perf_counter_ns()
+        r = V.route(idx, starts, cfg.num_experts)
+        if fp8:
+            dx, sc = V.dispatch_fp8(x, r["src_of_slot"], K)
+        else:
+            dx, sc = V.dispatch(x, r["src_of_slot"], K), None
+        t1 = time.perf_counter_ns()
+        ey = V.stub(dx, r["meta"], wl.stub_kind, cfg.num_experts, wl.world_size, cfg.out_dtype, scale=sc)
+        t2 = time.perf_counter_ns()
+        y_cpu = comb(ey, w, r["slot_of_entry"], cfg.out_dtype)
+        t3 = time.perf_counter_ns()
+        times.append(((t1 - t0) + (t3 - t2)) / 1e3)
+        if len(times) >= 3 and (time.perf_counter() - t_begin > budget_s or len(times) >= 50):
+            break
+    us = statistics.median(times[1:])
+    same = bool(torch.equal(y_gpu.cpu().view(torch.int16), y_cpu.view(torch.int16)))
+    return dict(value=round(b_dc / us / 1e3, 3), unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                dispatch_combine_us=round(us, 1),
+                sample=f"full workload {wl.name}: {len(times) - 1} timed passes of route+dispatch+combine "
+                       f"(vectorised torch-CPU oracle), median",
+                gpu_output_bit_identical=same)
+
+
+if __name__ == "__main__":
+    main()

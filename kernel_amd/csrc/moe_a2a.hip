@@ -378,6 +378,7 @@ __global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a
                                                                       uint4* __restrict__ disp, int nvec,
                                                                       int nsplit) {
   __shared__ int s_slot[MOE_A2A_MAX_TOPK];
+  __shared__ int s_key[MOE_A2A_MAX_TOPK];
   __shared__ int s_hist[MOE_A2A_MAX_EXPERTS];
   __shared__ int s_tmp[kRowThreads / kWave + 1];
   const int tid = threadIdx.x;
@@ -415,24 +416,42 @@ __global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a
     int c = c0 + u * kRowThreads;
     if (c < nvec) v[u] = src[c];
   }
-  if (tid < a.K) s_slot[tid] = 0;
+  if (tid < a.K) {  // keys of this token's own entries
+    int ik = t * a.K + tid;
+    s_key[tid] = (load_expert(a, ik, true) << 12) | ik;
+    s_slot[tid] = 0;
+  }
   __syncthreads();
 
   constexpr int kChunk = kRowThreads * kFusedEntriesPerThread;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(a.indices) & 15u) == 0;
   for (int i0 = 0; i0 < a.R; i0 += kChunk) {
     int key[kFusedEntriesPerThread];
     const int ibase = i0 + tid * kFusedEntriesPerThread;
+    if (vec_ok && ibase + kFusedEntriesPerThread <= a.R) {
+      const int4* p = reinterpret_cast<const int4*>(a.indices + ibase);
+      const int4 q0 = p[0], q1 = p[1];
+      const int e[kFusedEntriesPerThread] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
-    for (int m = 0; m < kFusedEntriesPerThread; ++m) {
-      int i = ibase + m;
-      bool valid = i < a.R;
-      int e = load_expert(a, i, valid);
-      key[m] = valid ? ((e << 12) | i) : 0x7fffffff;
+      for (int m = 0; m < kFusedEntriesPerThread; ++m) {
+        int em = e[m];
+        if (em < 0 || em >= a.E) {
+          if (a.status) *a.status = 1;
+          em = em < 0 ? 0 : a.E - 1;
+        }
+        key[m] = (em << 12) | (ibase + m);
+      }
+    } else {
+#pragma unroll
+      for (int m = 0; m < kFusedEntriesPerThread; ++m) {
+        int i = ibase + m;
+        bool valid = i < a.R;
+        int e = load_expert(a, i, valid);
+        key[m] = valid ? ((e << 12) | i) : 0x7fffffff;
+      }
     }
     for (int k = 0; k < a.K; ++k) {
-      int ik = t * a.K + k;
-      int ek = load_expert(a, ik, true);
-      int mykey = (ek << 12) | ik;
+      const int mykey = s_key[k];
       int c = 0;
 #pragma unroll
       for (int m = 0; m < kFusedEntriesPerThread; ++m) c += __popcll(__ballot(key[m] < mykey));
