@@ -74,7 +74,7 @@ def summarise(per):
                     median_us=round(statistics.median(v), 3), launches=len(v)) for k, v in per.items()}
 
 
-ROUTE_KERNELS = ("route_single", "route_hist", "route_scan", "route_rank")
+ROUTE_KERNELS = ("route_tiles", "route_hist", "route_scan", "route_rank")
 DISPATCH_KERNELS = ("dispatch_rows", "route_dispatch", "dispatch_fp8")
 COMBINE_KERNELS = ("combine_rows", "stub_combine")
 STUB_KERNELS = ("stub_rows", "stub_fp8")
@@ -171,7 +171,7 @@ def main():
         data="synthetic",
         config=dict(workload=args.workload, tokens=T, experts=E, top_k=K, hidden=H, emulated_ranks=W,
                     routed_rows=T * K, combine=args.combine, launch="hipGraph replay" if use_graph else "eager",
-                    fused_route=bool(not args.no_fuse_route and not fp8 and T * K <= lib.moe_a2a_fused_max_rows()),
+                    fused_route=bool(not args.no_fuse_route and not fp8 and lib.moe_a2a_fused_ok(T, K, H)),
                     fused_stub=bool(args.fuse_stub)),
         dispatch_combine_us=round(t_dc, 3), route_us=round(t_route, 3), dispatch_us=round(t_disp, 3),
         stub_us=round(t_stub, 3), combine_us=round(t_comb, 3),

@@ -104,6 +104,9 @@ int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, 
  * routing kernel has to finish first.  Outputs as moe_a2a_route + moe_a2a_dispatch.
  */
 int moe_a2a_fused_max_rows(void);
+/* 1 if moe_a2a_route_dispatch is the faster choice for this shape: it needs R within the limit
+ * above and a routing table small enough that re-reading it in every workgroup stays cheap. */
+int moe_a2a_fused_ok(int T, int K, int H);
 int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
                            int K, int E, int W, int H, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
                            int32_t* src_of_slot, int32_t* meta, int32_t* status, void* disp_x,

@@ -25,6 +25,7 @@ PROTOTYPES = {
                              _vp, C.c_size_t, _vp]),
     "moe_a2a_dispatch": (_int, [_vp, _i32p, _vp, _int, _int, _int, _vp]),
     "moe_a2a_fused_max_rows": (_int, []),
+    "moe_a2a_fused_ok": (_int, [_int, _int, _int]),
     "moe_a2a_route_dispatch": (_int, [_vp, _i32p, _i32p, _int, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p,
                                       _i32p, _i32p, _i32p, _vp, _vp]),
     "moe_a2a_dispatch_fp8": (_int, [_vp, _int, _i32p, _vp, _vp, _int, _int, _int, _vp]),

@@ -173,7 +173,9 @@ class HipAllToAll:
         lib, st = self.lib, _stream()
         route_out = (_ptr(b["counts"]), _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]),
                      _ptr(b["meta"]), _ptr(b["status"]))
-        if self.fuse_route and not self.fp8_dispatch and 0 < T * K <= self._fused_max_rows:
+        if self.fuse_route and not self.fp8_dispatch and (
+                self.fuse_route == "always" and 0 < T * K <= self._fused_max_rows
+                or self.lib.moe_a2a_fused_ok(T, K, H)):
             _lib.check(lib.moe_a2a_route_dispatch(_ptr(dp_x), _ptr(indices), _ptr(rank_start), self.rank, T, K, E, W,
                                                   H, *route_out, _ptr(b["disp_x"]), st), "moe_a2a_route_dispatch")
         else:

@@ -23,13 +23,16 @@ namespace {
 constexpr int kWave = 64;
 constexpr int kRouteThreads = 1024;
 constexpr int kRouteWaves = kRouteThreads / kWave;
-constexpr int kRouteSingleMaxRows = 16 * kRouteThreads;  // one-workgroup routing up to here
-constexpr int kRowThreads = 256;
-constexpr int kFusedMaxRows = 4096;  // route_dispatch: 12-bit entry ids
-constexpr int kFusedEntriesPerThread = 8;
+constexpr int kRouteTilesMaxRows = 16 * kRouteThreads;  // one-launch routing up to here
+constexpr int kRowMaxThreads = 512;
+constexpr int kFusedIdBits = 13;
+constexpr int kFusedMaxRows = 1 << kFusedIdBits;  // route_dispatch packs (expert, entry id) into one key
+constexpr int kFusedEntriesPerThread = 4;
+constexpr int kFusedMaxThreads = 1024;
+constexpr long long kFusedMaxTableReads = 1ll << 20;  // entries read by all workgroups together
 
 enum KernelId {
-  KID_ROUTE_SINGLE = 0,
+  KID_ROUTE_TILES = 0,
   KID_ROUTE_HIST,
   KID_ROUTE_SCAN,
   KID_ROUTE_RANK,
@@ -43,7 +46,7 @@ enum KernelId {
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
-    "route_single", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch",
+    "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine"};
 
 // ---------------------------------------------------------------------------------------
@@ -220,58 +223,58 @@ __device__ __forceinline__ int tile_wave_counts(int* wcnt, int E, int e, bool va
   return rank;
 }
 
-// Whole routing in one workgroup: pass 1 histogram + scan, pass 2 stable ranks tile by tile.
-__global__ __launch_bounds__(kRouteThreads) void route_single_kernel(RouteArgs a) {
+// Routing in ONE launch for up to kRouteTilesMaxRows entries.  A tile is kRouteThreads
+// consecutive entries and has its own workgroup.  Every workgroup counts, in LDS, the rows of
+// each expert in the tiles before its own and in the rest of the table (it reads the whole
+// routing table: R * 4 bytes per workgroup, which is what replaces a histogram launch, a scan
+// launch and the round trips between them), scans the totals into offsets, ranks its own
+// entries stably (wave match + per-wave counts) and writes their slots and meta rows.
+__global__ __launch_bounds__(kRouteThreads) void route_tiles_kernel(RouteArgs a) {
   extern __shared__ int smem[];
   int* wcnt = smem;
-  int* base = wcnt + kRouteWaves * a.E;
-  int* tmp = base + a.E;
+  int* before = wcnt + kRouteWaves * a.E;
+  int* rest = before + a.E;
+  int* tmp = rest + a.E;
   int* starts = tmp + kRouteWaves + 1;
   const int tid = threadIdx.x;
+  const int tile_lo = blockIdx.x * kRouteThreads;
   load_starts(a, starts);
-  for (int j = tid; j < a.E; j += kRouteThreads) base[j] = 0;
+  for (int j = tid; j < 2 * a.E; j += kRouteThreads) before[j] = 0;  // before[] and rest[] are adjacent
   __syncthreads();
-  for (int i0 = 0; i0 < a.R; i0 += kRouteThreads) {
-    int i = i0 + tid;
-    bool valid = i < a.R;
-    int e = load_expert(a, i, valid);
-    int rank, cnt;
-    wave_match(e, valid, a.nbits, rank, cnt);
-    if (valid && rank == 0) atomicAdd(&base[e], cnt);  // LDS counter; order does not matter for a sum
+#pragma unroll 4
+  for (int i = tid; i < a.R; i += kRouteThreads) {
+    int e = load_expert(a, i, true);
+    atomicAdd(i < tile_lo ? &before[e] : &rest[e], 1);  // LDS counters; a sum does not depend on order
   }
-  __syncthreads();
-  int v = tid < a.E ? base[tid] : 0;
+  const int i = tile_lo + tid;
+  const bool valid = i < a.R;
+  const int e = load_expert(a, i, valid);
+  const int rank = tile_wave_counts(wcnt, a.E, e, valid, a.nbits);  // its barriers also cover the counters
+  const int all = tid < a.E ? before[tid] + rest[tid] : 0;
   int total;
-  int excl = block_exclusive_scan(v, tmp, total);
-  if (tid < a.E) {
-    base[tid] = excl;
-    a.counts[tid] = v;
-    a.offsets[tid] = excl;
-  }
-  if (tid == 0) a.offsets[a.E] = total;
-  __syncthreads();
-  for (int i0 = 0; i0 < a.R; i0 += kRouteThreads) {
-    int i = i0 + tid;
-    bool valid = i < a.R;
-    int e = load_expert(a, i, valid);
-    int rank = tile_wave_counts(wcnt, a.E, e, valid, a.nbits);
+  const int excl = block_exclusive_scan(all, tmp, total);
+  if (blockIdx.x == 0) {
     if (tid < a.E) {
-      int run = base[tid];
-      for (int w = 0; w < kRouteWaves; ++w) {
-        int c = wcnt[w * a.E + tid];
-        wcnt[w * a.E + tid] = run;
-        run += c;
-      }
-      base[tid] = run;
+      a.counts[tid] = all;
+      a.offsets[tid] = excl;
     }
-    __syncthreads();
-    if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank);
-    __syncthreads();
+    if (tid == 0) a.offsets[a.E] = total;
   }
+  if (tid < a.E) {
+    int run = excl + before[tid];
+    for (int w = 0; w < kRouteWaves; ++w) {
+      int c = wcnt[w * a.E + tid];
+      wcnt[w * a.E + tid] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank);
 }
 
-// Multi-workgroup routing, step 1: rows per (expert, tile), expert-major.
-__global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(RouteArgs a, int32_t* tile_hist, int ntiles) {
+// Routing in three launches for larger tables.
+// step 1: rows per (tile, expert), tile-major so that lane e reads and writes coalesced.
+__global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(RouteArgs a, int32_t* tile_hist) {
   extern __shared__ int smem[];
   int* wcnt = smem;
   const int tid = threadIdx.x;
@@ -279,43 +282,65 @@ __global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(RouteArgs a, 
   bool valid = i < a.R;
   int e = load_expert(a, i, valid);
   tile_wave_counts(wcnt, a.E, e, valid, a.nbits);
-  for (int j = tid; j < a.E; j += kRouteThreads) {
+  if (tid < a.E) {
     int s = 0;
-    for (int w = 0; w < kRouteWaves; ++w) s += wcnt[w * a.E + j];
-    tile_hist[(size_t)j * ntiles + blockIdx.x] = s;
+    for (int w = 0; w < kRouteWaves; ++w) s += wcnt[w * a.E + tid];
+    tile_hist[(size_t)blockIdx.x * a.E + tid] = s;
   }
 }
 
-// step 2: exclusive scan of the (expert, tile) matrix in place, counts and offsets.
-__global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int32_t* tile_hist, int n, int E, int ntiles,
+// step 2: every count becomes the number of rows of its expert in earlier tiles, and the
+// column totals are scanned into counts and offsets.  One workgroup; floor(1024 / E) threads
+// share a column, each walking a contiguous range of tiles eight loads at a time.
+__global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int32_t* tile_hist, int E, int ntiles,
                                                                     int32_t* counts, int32_t* offsets) {
+  __shared__ int part_sum[kRouteThreads];
   __shared__ int tmp[kRouteWaves + 1];
   const int tid = threadIdx.x;
-  int per = (n + kRouteThreads - 1) / kRouteThreads;
-  int lo = tid * per;
-  int hi = min(lo + per, n);
-  int s = 0;
-  for (int j = lo; j < hi; ++j) s += tile_hist[j];
-  int total;
-  int run = block_exclusive_scan(s, tmp, total);
-  for (int j = lo; j < hi; ++j) {
-    int c = tile_hist[j];
-    tile_hist[j] = run;
-    run += c;
+  const int parts = kRouteThreads / E;  // >= 1 because E <= 1024
+  const int p = tid / E, e = tid - p * E;
+  const bool live = p < parts;
+  const int span = (ntiles + parts - 1) / parts;
+  const int lo = min(p * span, ntiles), hi = live ? min(lo + span, ntiles) : lo;
+  int sum = 0;
+  for (int b0 = lo; b0 < hi; b0 += 8) {
+    int c[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) c[u] = b0 + u < hi ? tile_hist[(size_t)(b0 + u) * E + e] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sum += c[u];
   }
+  part_sum[tid] = live ? sum : 0;
   __syncthreads();
-  for (int e = tid; e < E; e += kRouteThreads) {
-    int first = tile_hist[(size_t)e * ntiles];
-    int next = e + 1 < E ? tile_hist[(size_t)(e + 1) * ntiles] : total;
-    offsets[e] = first;
-    counts[e] = next - first;
+  int run = 0, column = 0;
+  if (live)
+    for (int q = 0; q < parts; ++q) {
+      int v = part_sum[q * E + e];
+      if (q < p) run += v;
+      column += v;
+    }
+  for (int b0 = lo; b0 < hi; b0 += 8) {
+    int c[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) c[u] = b0 + u < hi ? tile_hist[(size_t)(b0 + u) * E + e] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (b0 + u < hi) tile_hist[(size_t)(b0 + u) * E + e] = run;
+      run += c[u];
+    }
+  }
+  const bool first = live && p == 0;  // tid == e
+  int total;
+  int excl = block_exclusive_scan(first ? column : 0, tmp, total);
+  if (first) {
+    counts[e] = column;
+    offsets[e] = excl;
   }
   if (tid == 0) offsets[E] = total;
 }
 
-// step 3: stable rank inside the tile + first slot of (expert, tile).
-__global__ __launch_bounds__(kRouteThreads) void route_rank_kernel(RouteArgs a, const int32_t* tile_base,
-                                                                    int ntiles) {
+// step 3: stable rank inside the tile + first slot of (expert, tile) from steps 1 and 2.
+__global__ __launch_bounds__(kRouteThreads) void route_rank_kernel(RouteArgs a, const int32_t* tile_hist) {
   extern __shared__ int smem[];
   int* wcnt = smem;
   int* starts = wcnt + kRouteWaves * a.E;
@@ -325,11 +350,11 @@ __global__ __launch_bounds__(kRouteThreads) void route_rank_kernel(RouteArgs a, 
   bool valid = i < a.R;
   int e = load_expert(a, i, valid);
   int rank = tile_wave_counts(wcnt, a.E, e, valid, a.nbits);
-  for (int j = tid; j < a.E; j += kRouteThreads) {
-    int run = tile_base[(size_t)j * ntiles + blockIdx.x];
+  if (tid < a.E) {
+    int run = a.offsets[tid] + tile_hist[(size_t)blockIdx.x * a.E + tid];
     for (int w = 0; w < kRouteWaves; ++w) {
-      int c = wcnt[w * a.E + j];
-      wcnt[w * a.E + j] = run;
+      int c = wcnt[w * a.E + tid];
+      wcnt[w * a.E + tid] = run;
       run += c;
     }
   }
@@ -338,60 +363,100 @@ __global__ __launch_bounds__(kRouteThreads) void route_rank_kernel(RouteArgs a, 
 }
 
 // ---------------------------------------------------------------------------------------
+// row kernels: geometry and memory helpers
+// ---------------------------------------------------------------------------------------
+// A row of nvec 16-byte vectors is cut into nsplit equal column ranges of `per` vectors; one
+// workgroup of round_up(per, 64) <= 512 threads moves one range, one vector per lane, so no
+// lane idles when nvec is a multiple of 64 (H = 7168 -> two workgroups of 448 lanes).
+//
+// Cache policy of the row traffic (rows are produced by one kernel and consumed by a later
+// one, never re-read by the kernel that touches them):
+//   STREAM = 0  working set fits the caches: plain loads; stores write through (sc0 sc1) so
+//               the lines leave L2 while the kernel runs instead of in its end-of-kernel
+//               write-back;
+//   STREAM = 1  working set far beyond the 256 MB Infinity Cache: non-temporal loads and
+//               stores, which keep streamed rows from evicting each other.
+// Scattered row stores of the dispatch always write through.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void store_through(uint4* p, const uint4& v) {
+  u32x4_t t = {v.x, v.y, v.z, v.w};
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(t) : "memory");
+}
+
+template <int STREAM>
+__device__ __forceinline__ void store_row(uint4* p, const uint4& v) {
+  if (STREAM) {
+    u32x4_t t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4_t*>(p));
+  } else {
+    store_through(p, v);
+  }
+}
+
+template <int STREAM>
+__device__ __forceinline__ uint4 load_row(const uint4* p) {
+  if (STREAM) {
+    u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return make_uint4(t.x, t.y, t.z, t.w);
+  }
+  return *p;
+}
+
+struct RowCut {
+  int t;        // row handled by this workgroup
+  int c;        // vector index inside the row
+  bool active;  // lane has a vector
+};
+
+__device__ __forceinline__ RowCut row_cut(int nvec, int per, int nsplit) {
+  RowCut r;
+  r.t = blockIdx.x / nsplit;
+  const int cs = blockIdx.x - r.t * nsplit;
+  r.c = cs * per + threadIdx.x;
+  r.active = (int)threadIdx.x < per && r.c < nvec;
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------
 // dispatch: token row -> K rows
 // ---------------------------------------------------------------------------------------
-// One workgroup copies U*256 16-byte vectors of one token row to that token's K slots.
-template <int U>
-__global__ __launch_bounds__(kRowThreads) void dispatch_rows_kernel(const uint4* __restrict__ x,
-                                                                     const int32_t* __restrict__ slot_of_entry,
-                                                                     uint4* __restrict__ disp, int K, int nvec,
-                                                                     int nsplit) {
-  const int t = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - t * nsplit;
-  const int c0 = cs * (kRowThreads * U) + threadIdx.x;
-  const uint4* src = x + (size_t)t * nvec;
-  uint4 v[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    int c = c0 + u * kRowThreads;
-    if (c < nvec) v[u] = src[c];
-  }
-  const int32_t* sl = slot_of_entry + (size_t)t * K;
-  for (int k = 0; k < K; ++k) {
-    uint4* dst = disp + (size_t)sl[k] * nvec;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      int c = c0 + u * kRowThreads;
-      if (c < nvec) dst[c] = v[u];
-    }
-  }
+template <int STREAM>
+__global__ __launch_bounds__(kRowMaxThreads) void dispatch_rows_kernel(const uint4* __restrict__ x,
+                                                                        const int32_t* __restrict__ slot_of_entry,
+                                                                        uint4* __restrict__ disp, int K, int nvec,
+                                                                        int per, int nsplit) {
+  const RowCut r = row_cut(nvec, per, nsplit);
+  if (!r.active) return;
+  const uint4 v = load_row<STREAM>(x + (size_t)r.t * nvec + r.c);
+  const int32_t* sl = slot_of_entry + (size_t)r.t * K;
+  for (int k = 0; k < K; ++k) store_through(disp + (size_t)sl[k] * nvec + r.c, v);
 }
 
 // Routing folded into the dispatch for R <= kFusedMaxRows.  The slot of entry i is the number
 // of entries whose (expert, entry id) pair is smaller, so a workgroup can find the K slots of
 // its own token by comparing every entry of the table against K keys: each lane holds
 // kFusedEntriesPerThread entries, a ballot + popcount per (entry, key) counts a wave's share,
-// and LDS counters add the waves up.  Column split 0 of each token also writes the index
-// arrays and meta rows; one extra workgroup writes counts and offsets.
-template <int U>
-__global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a, const uint4* __restrict__ x,
-                                                                      uint4* __restrict__ disp, int nvec,
-                                                                      int nsplit) {
+// and LDS counters add the waves up.  The row load is issued first and is in flight meanwhile.
+// Column split 0 of each token also writes the index arrays and meta rows; workgroup 0
+// writes counts and offsets.
+__global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteArgs a, const uint4* __restrict__ x,
+                                                                         uint4* __restrict__ disp, int nvec,
+                                                                         int per, int nsplit) {
   __shared__ int s_slot[MOE_A2A_MAX_TOPK];
-  __shared__ int s_key[MOE_A2A_MAX_TOPK];
   __shared__ int s_hist[MOE_A2A_MAX_EXPERTS];
-  __shared__ int s_tmp[kRowThreads / kWave + 1];
+  __shared__ int s_tmp[kFusedMaxThreads / kWave + 1];
   const int tid = threadIdx.x;
+  const int nthreads = blockDim.x;
   const int lane = tid & (kWave - 1);
-  const int ntok_blocks = a.T * nsplit;
 
-  if ((int)blockIdx.x == ntok_blocks) {  // counts + offsets
-    for (int j = tid; j < a.E; j += kRowThreads) s_hist[j] = 0;
+  if (blockIdx.x == 0) {  // counts + offsets
+    for (int j = tid; j < a.E; j += nthreads) s_hist[j] = 0;
     __syncthreads();
-    for (int i = tid; i < a.R; i += kRowThreads) atomicAdd(&s_hist[load_expert(a, i, true)], 1);
+    for (int i = tid; i < a.R; i += nthreads) atomicAdd(&s_hist[load_expert(a, i, true)], 1);
     __syncthreads();
-    const int per = (a.E + kRowThreads - 1) / kRowThreads;
-    int lo = min(tid * per, a.E), hi = min(lo + per, a.E);
+    const int span = (a.E + nthreads - 1) / nthreads;
+    int lo = min(tid * span, a.E), hi = min(lo + span, a.E);
     int s = 0;
     for (int j = lo; j < hi; ++j) s += s_hist[j];
     int total;
@@ -406,32 +471,29 @@ __global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a
     return;
   }
 
-  const int t = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - t * nsplit;
-  const int c0 = cs * (kRowThreads * U) + tid;
-  const uint4* src = x + (size_t)t * nvec;
-  uint4 v[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {  // row loads are in flight while the slots are worked out
-    int c = c0 + u * kRowThreads;
-    if (c < nvec) v[u] = src[c];
+  // every load this workgroup needs is issued here, before anything waits
+  const int t = (blockIdx.x - 1) / nsplit;
+  const int cs = (blockIdx.x - 1) - t * nsplit;
+  const int c = cs * per + tid;
+  const bool active = tid < per && c < nvec;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (active) v = x[(size_t)t * nvec + c];
+  int ownkey = 0x7fffffff;  // lane k of every wave: key of the token's k-th entry
+  if (lane < a.K) {
+    int ik = t * a.K + lane;
+    ownkey = (load_expert(a, ik, true) << kFusedIdBits) | ik;
   }
-  if (tid < a.K) {  // keys of this token's own entries
-    int ik = t * a.K + tid;
-    s_key[tid] = (load_expert(a, ik, true) << 12) | ik;
-    s_slot[tid] = 0;
-  }
-  __syncthreads();
+  if (tid < a.K) s_slot[tid] = 0;
 
-  constexpr int kChunk = kRowThreads * kFusedEntriesPerThread;
+  const int chunk = nthreads * kFusedEntriesPerThread;
   const bool vec_ok = (reinterpret_cast<uintptr_t>(a.indices) & 15u) == 0;
-  for (int i0 = 0; i0 < a.R; i0 += kChunk) {
+  bool zeroed = false;
+  for (int i0 = 0; i0 < a.R; i0 += chunk) {
     int key[kFusedEntriesPerThread];
     const int ibase = i0 + tid * kFusedEntriesPerThread;
     if (vec_ok && ibase + kFusedEntriesPerThread <= a.R) {
-      const int4* p = reinterpret_cast<const int4*>(a.indices + ibase);
-      const int4 q0 = p[0], q1 = p[1];
-      const int e[kFusedEntriesPerThread] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+      const int4 q0 = *reinterpret_cast<const int4*>(a.indices + ibase);
+      const int e[kFusedEntriesPerThread] = {q0.x, q0.y, q0.z, q0.w};
 #pragma unroll
       for (int m = 0; m < kFusedEntriesPerThread; ++m) {
         int em = e[m];
@@ -439,7 +501,7 @@ __global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a
           if (a.status) *a.status = 1;
           em = em < 0 ? 0 : a.E - 1;
         }
-        key[m] = (em << 12) | (ibase + m);
+        key[m] = (em << kFusedIdBits) | (ibase + m);
       }
     } else {
 #pragma unroll
@@ -447,31 +509,29 @@ __global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a
         int i = ibase + m;
         bool valid = i < a.R;
         int e = load_expert(a, i, valid);
-        key[m] = valid ? ((e << 12) | i) : 0x7fffffff;
+        key[m] = valid ? ((e << kFusedIdBits) | i) : 0x7fffffff;
       }
     }
+    if (!zeroed) {
+      __syncthreads();  // counters are zero before the first add
+      zeroed = true;
+    }
+    if (__ballot(ibase < a.R) == 0) continue;  // this wave holds no entries of the chunk
     for (int k = 0; k < a.K; ++k) {
-      const int mykey = s_key[k];
-      int c = 0;
+      const int mykey = __builtin_amdgcn_readlane(ownkey, k);
+      int cnt = 0;
 #pragma unroll
-      for (int m = 0; m < kFusedEntriesPerThread; ++m) c += __popcll(__ballot(key[m] < mykey));
-      if (lane == 0 && c) atomicAdd(&s_slot[k], c);
+      for (int m = 0; m < kFusedEntriesPerThread; ++m) cnt += __popcll(__ballot(key[m] < mykey));
+      if (lane == 0 && cnt) atomicAdd(&s_slot[k], cnt);
     }
   }
   __syncthreads();
 
-  for (int k = 0; k < a.K; ++k) {
-    uint4* dst = disp + (size_t)s_slot[k] * nvec;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      int c = c0 + u * kRowThreads;
-      if (c < nvec) dst[c] = v[u];
-    }
-  }
+  if (active)
+    for (int k = 0; k < a.K; ++k) store_through(disp + (size_t)s_slot[k] * nvec + c, v);
   if (cs == 0 && tid < a.K) {
-    int i = t * a.K + tid;
-    int e = load_expert(a, i, true);
-    int slot = s_slot[tid];
+    const int i = t * a.K + tid;
+    const int slot = s_slot[tid];
     a.slot_of_entry[i] = slot;
     a.src_of_slot[slot] = i;
     int sr = a.src_rank, tl = t;
@@ -485,7 +545,7 @@ __global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a
       tl = t - a.rank_start[lo];
     }
     int32_t* m = a.meta + (size_t)slot * MOE_A2A_META_DIM;
-    m[0] = e;
+    m[0] = ownkey >> kFusedIdBits;
     m[1] = sr;
     m[2] = tl;
     m[3] = tid;
@@ -495,22 +555,18 @@ __global__ __launch_bounds__(kRowThreads) void route_dispatch_kernel(RouteArgs a
 
 // fp8 dispatch.  8 lanes own one 128-column block (16 elements each): block amax by three
 // xor-shuffles, scale = amax/448, q = e4m3(x/scale) with the hardware conversion (RNE).
-template <class E>
-__global__ __launch_bounds__(kRowThreads) void dispatch_fp8_kernel(const uint4* __restrict__ x,
-                                                                    const int32_t* __restrict__ slot_of_entry,
-                                                                    uint4* __restrict__ disp_q,
-                                                                    float* __restrict__ disp_scale, int K, int nblk,
-                                                                    int nsplit) {
-  constexpr int kBlocksPerWg = kRowThreads / 8;
-  const int t = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - t * nsplit;
-  const int gb = cs * kBlocksPerWg + (threadIdx.x >> 3);
-  const int sub = threadIdx.x & 7;
-  const bool valid = gb < nblk;
+// Geometry is in lanes of 16 input elements: nvec = 8 * nblk, per a multiple of 8.
+template <class E, int STREAM>
+__global__ __launch_bounds__(kRowMaxThreads) void dispatch_fp8_kernel(const uint4* __restrict__ x,
+                                                                       const int32_t* __restrict__ slot_of_entry,
+                                                                       uint4* __restrict__ disp_q,
+                                                                       float* __restrict__ disp_scale, int K,
+                                                                       int nblk, int per, int nsplit) {
+  const RowCut r = row_cut(nblk * 8, per, nsplit);
   float f[16];
-  if (valid) {
-    const uint4* src = x + ((size_t)t * nblk + gb) * 16 + sub * 2;
-    uint4 v0 = src[0], v1 = src[1];
+  if (r.active) {
+    const uint4* src = x + ((size_t)r.t * nblk * 8 + r.c) * 2;
+    uint4 v0 = load_row<STREAM>(src), v1 = load_row<STREAM>(src + 1);
     uint32_t d[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -527,7 +583,8 @@ __global__ __launch_bounds__(kRowThreads) void dispatch_fp8_kernel(const uint4* 
   amax = fmaxf(amax, __shfl_xor(amax, 1, kWave));
   amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
   amax = fmaxf(amax, __shfl_xor(amax, 4, kWave));
-  float scale = amax == 0.f ? 1.f : amax / 448.f;
+  if (!r.active) return;
+  const float scale = amax == 0.f ? 1.f : amax / 448.f;
   uint32_t q[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -535,50 +592,30 @@ __global__ __launch_bounds__(kRowThreads) void dispatch_fp8_kernel(const uint4* 
     w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * j + 2] / scale, f[4 * j + 3] / scale, w, true);
     q[j] = (uint32_t)w;
   }
-  if (!valid) return;
   const uint4 qv = make_uint4(q[0], q[1], q[2], q[3]);
-  const int32_t* sl = slot_of_entry + (size_t)t * K;
+  const int gb = r.c >> 3;
+  const int32_t* sl = slot_of_entry + (size_t)r.t * K;
   for (int k = 0; k < K; ++k) {
     size_t row = (size_t)sl[k];
-    disp_q[(row * nblk + gb) * 8 + sub] = qv;
-    if (sub == 0) disp_scale[row * nblk + gb] = scale;
+    store_through(disp_q + row * nblk * 8 + r.c, qv);
+    if ((r.c & 7) == 0) disp_scale[row * nblk + gb] = scale;
   }
 }
 
 // ---------------------------------------------------------------------------------------
 // expert stub
 // ---------------------------------------------------------------------------------------
-template <class In, class Out, int U>
-__global__ __launch_bounds__(kRowThreads) void stub_rows_kernel(const uint4* __restrict__ disp,
-                                                                 const int32_t* __restrict__ meta,
-                                                                 uint4* __restrict__ y, int stub_kind, int E,
-                                                                 int E_l, int nvec, int nsplit) {
-  const int row = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - row * nsplit;
-  const int c0 = cs * (kRowThreads * U) + threadIdx.x;
-  const float s = stub_factor(meta[(size_t)row * MOE_A2A_META_DIM], stub_kind, E, E_l);
-  const uint4* src = disp + (size_t)row * nvec;
-  uint4* dst = y + (size_t)row * nvec;
-  uint4 v[U];
+template <class In, class Out>
+__device__ __forceinline__ uint4 stub_vec(const uint4& v, float s) {
+  uint32_t d[4];
+  unpack8(v, d);
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    int c = c0 + u * kRowThreads;
-    if (c < nvec) v[u] = src[c];
+  for (int j = 0; j < 4; ++j) {
+    float a = In::lo(d[j]), b = In::hi(d[j]);
+    round_pair<Out>(a, b);  // .to(out_dtype); identity when In == Out
+    d[j] = Out::pack(a * s, b * s);
   }
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    int c = c0 + u * kRowThreads;
-    if (c >= nvec) continue;
-    uint32_t d[4];
-    unpack8(v[u], d);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float a = In::lo(d[j]), b = In::hi(d[j]);
-      round_pair<Out>(a, b);  // .to(out_dtype)
-      d[j] = Out::pack(a * s, b * s);
-    }
-    dst[c] = make_uint4(d[0], d[1], d[2], d[3]);
-  }
+  return make_uint4(d[0], d[1], d[2], d[3]);
 }
 
 __device__ __forceinline__ void fp8x4_to_f32(uint32_t w, float (&f)[4]) {
@@ -588,20 +625,9 @@ __device__ __forceinline__ void fp8x4_to_f32(uint32_t w, float (&f)[4]) {
   f[3] = __builtin_amdgcn_cvt_f32_fp8((int)w, 3);
 }
 
-// fp8 rows: each lane turns 16 bytes into 16 output elements (two 16-byte stores).
+// 16 fp8 values -> 16 values of Out: round_out((f32(q) * scale) * s)
 template <class Out>
-__global__ __launch_bounds__(kRowThreads) void stub_fp8_kernel(const uint4* __restrict__ disp_q,
-                                                                const float* __restrict__ disp_scale,
-                                                                const int32_t* __restrict__ meta,
-                                                                uint4* __restrict__ y, int stub_kind, int E, int E_l,
-                                                                int nblk, int nsplit) {
-  const int row = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - row * nsplit;
-  const int c = cs * kRowThreads + threadIdx.x;  // 16-byte vector of the fp8 row
-  if (c >= nblk * 8) return;
-  const float s = stub_factor(meta[(size_t)row * MOE_A2A_META_DIM], stub_kind, E, E_l);
-  const float scale = disp_scale[(size_t)row * nblk + (c >> 3)];
-  const uint4 q = disp_q[(size_t)row * nblk * 8 + c];
+__device__ __forceinline__ void stub_vec_fp8(const uint4& q, float scale, float s, uint4& o0, uint4& o1) {
   const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
   uint32_t o[8];
 #pragma unroll
@@ -611,32 +637,103 @@ __global__ __launch_bounds__(kRowThreads) void stub_fp8_kernel(const uint4* __re
     o[2 * j] = Out::pack((f[0] * scale) * s, (f[1] * scale) * s);
     o[2 * j + 1] = Out::pack((f[2] * scale) * s, (f[3] * scale) * s);
   }
-  uint4* dst = y + ((size_t)row * nblk * 8 + c) * 2;
-  dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
-  dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+  o0 = make_uint4(o[0], o[1], o[2], o[3]);
+  o1 = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
+template <class In, class Out, int STREAM>
+__global__ __launch_bounds__(kRowMaxThreads) void stub_rows_kernel(const uint4* __restrict__ disp,
+                                                                    const int32_t* __restrict__ meta,
+                                                                    uint4* __restrict__ y, int stub_kind, int E,
+                                                                    int E_l, int nvec, int per, int nsplit) {
+  const RowCut r = row_cut(nvec, per, nsplit);
+  if (!r.active) return;
+  const uint4 v = load_row<STREAM>(disp + (size_t)r.t * nvec + r.c);
+  const float s = stub_factor(meta[(size_t)r.t * MOE_A2A_META_DIM], stub_kind, E, E_l);
+  store_row<STREAM>(y + (size_t)r.t * nvec + r.c, stub_vec<In, Out>(v, s));
+}
+
+// fp8 rows: each lane turns 8 bytes into 8 output elements, so a wave's stores are one
+// contiguous kilobyte (a 16-byte load per lane would leave every lane two stores 32 bytes
+// apart).  Geometry is that of the 16-bit output row: nvec = H / 8 lanes.
+template <class Out, int STREAM>
+__global__ __launch_bounds__(kRowMaxThreads) void stub_fp8_kernel(const uint2* __restrict__ disp_q,
+                                                                   const float* __restrict__ disp_scale,
+                                                                   const int32_t* __restrict__ meta,
+                                                                   uint4* __restrict__ y, int stub_kind, int E,
+                                                                   int E_l, int nvec, int per, int nsplit) {
+  const RowCut r = row_cut(nvec, per, nsplit);
+  if (!r.active) return;
+  const uint2* src = disp_q + (size_t)r.t * nvec + r.c;
+  uint2 q;
+  if (STREAM) {
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    u32x2_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(src));
+    q = make_uint2(t.x, t.y);
+  } else {
+    q = *src;
+  }
+  const float scale = disp_scale[(size_t)r.t * (nvec >> 4) + (r.c >> 4)];
+  const float s = stub_factor(meta[(size_t)r.t * MOE_A2A_META_DIM], stub_kind, E, E_l);
+  float f0[4], f1[4];
+  fp8x4_to_f32(q.x, f0);
+  fp8x4_to_f32(q.y, f1);
+  store_row<STREAM>(y + (size_t)r.t * nvec + r.c,
+                    make_uint4(Out::pack((f0[0] * scale) * s, (f0[1] * scale) * s),
+                               Out::pack((f0[2] * scale) * s, (f0[3] * scale) * s),
+                               Out::pack((f1[0] * scale) * s, (f1[1] * scale) * s),
+                               Out::pack((f1[2] * scale) * s, (f1[3] * scale) * s)));
 }
 
 // ---------------------------------------------------------------------------------------
 // combine
 // ---------------------------------------------------------------------------------------
-// Order the K entries of token t for the weighted sum: STRICT = ascending slot (the order in
-// which the reference's receive loop meets them), F32 = k order.
-__device__ __forceinline__ void order_entries(const int32_t* __restrict__ slot_of_entry,
-                                              const float* __restrict__ weights, int t, int K, int mode,
-                                              int* s_slot, float* s_w, int* s_k) {
-  if ((int)threadIdx.x < K) {
-    const int32_t* sl = slot_of_entry + (size_t)t * K;
-    int mine = sl[threadIdx.x];
-    int pos = threadIdx.x;
-    if (mode == MOE_A2A_COMBINE_STRICT) {
-      pos = 0;
-      for (int j = 0; j < K; ++j) pos += sl[j] < mine;
-    }
-    s_slot[pos] = mine;
-    s_w[pos] = weights[(size_t)t * K + threadIdx.x];
-    s_k[pos] = threadIdx.x;
+// The K entries of a token are folded in STRICT = ascending slot order (the order in which the
+// reference's receive loop meets them) or F32 = k order.  Every wave keeps its own copy of the
+// token's entries, one per lane (lane k = entry k), ranks them with lane reads, and pulls the
+// entry at sorted position j into uniform registers -- no LDS, no barrier.
+struct EntryLanes {
+  int slot;   // lane k: slot of entry k
+  float w;    // lane k: routing weight of entry k
+  float f;    // lane k: stub factor of entry k (stub_combine only)
+  int pos;    // lane k: position of entry k in the fold order
+  bool live;  // lane < K
+};
+
+template <int MODE>
+__device__ __forceinline__ EntryLanes load_entries(const int32_t* __restrict__ slot_of_entry,
+                                                   const float* __restrict__ weights, int t, int K) {
+  const int lane = threadIdx.x & (kWave - 1);
+  EntryLanes en;
+  en.live = lane < K;
+  en.slot = 0x7fffffff;
+  en.w = 0.f;
+  en.f = 1.f;
+  if (en.live) {
+    en.slot = slot_of_entry[(size_t)t * K + lane];
+    en.w = weights[(size_t)t * K + lane];
   }
-  __syncthreads();
+  en.pos = lane;
+  if (MODE == MOE_A2A_COMBINE_STRICT) {
+    en.pos = 0;
+    for (int j = 0; j < K; ++j) {
+      const int sj = __builtin_amdgcn_readlane(en.slot, j);
+      en.pos += sj < en.slot || (sj == en.slot && j < lane);  // ties by k keep positions distinct
+    }
+  }
+  return en;
+}
+
+// value of x in lane `src` (uniform), as bits: the builtin takes integers
+__device__ __forceinline__ float lane_read(float x, int src) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src));
+}
+
+// lane that holds the entry of fold position j (uniform)
+template <int MODE>
+__device__ __forceinline__ int entry_lane(const EntryLanes& en, int j) {
+  if (MODE != MOE_A2A_COMBINE_STRICT) return j;
+  return __builtin_amdgcn_readfirstlane(__ffsll((long long)__ballot(en.live && en.pos == j)) - 1);
 }
 
 template <class E, int MODE>
@@ -653,134 +750,129 @@ __device__ __forceinline__ void accumulate8(float (&acc)[8], const uint4& v, flo
   }
 }
 
-template <class E, int MODE>
-__global__ __launch_bounds__(kRowThreads) void combine_rows_kernel(const uint4* __restrict__ y,
-                                                                    const float* __restrict__ weights,
-                                                                    const int32_t* __restrict__ slot_of_entry,
-                                                                    uint4* __restrict__ out, int K, int nvec,
-                                                                    int nsplit) {
-  __shared__ int s_slot[MOE_A2A_MAX_TOPK];
-  __shared__ float s_w[MOE_A2A_MAX_TOPK];
-  __shared__ int s_k[MOE_A2A_MAX_TOPK];
-  const int t = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - t * nsplit;
-  order_entries(slot_of_entry, weights, t, K, MODE, s_slot, s_w, s_k);
-  const int c = cs * kRowThreads + threadIdx.x;
-  if (c >= nvec) return;
+template <class E>
+__device__ __forceinline__ uint4 pack8(const float (&acc)[8]) {
+  return make_uint4(E::pack(acc[0], acc[1]), E::pack(acc[2], acc[3]), E::pack(acc[4], acc[5]),
+                    E::pack(acc[6], acc[7]));
+}
+
+// KT > 0: top-k known at compile time, all KT row loads of a lane are issued back to back.
+// KT == 0: any K, rows in batches of four.
+template <class E, int MODE, int KT, int STREAM>
+__global__ __launch_bounds__(kRowMaxThreads) void combine_rows_kernel(const uint4* __restrict__ y,
+                                                                       const float* __restrict__ weights,
+                                                                       const int32_t* __restrict__ slot_of_entry,
+                                                                       uint4* __restrict__ out, int K, int nvec,
+                                                                       int per, int nsplit) {
+  constexpr int kBatch = KT > 0 ? KT : 4;
+  const int k_rt = KT ? KT : K;
+  const RowCut r = row_cut(nvec, per, nsplit);
+  const EntryLanes en = load_entries<MODE>(slot_of_entry, weights, r.t, k_rt);
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  for (int j0 = 0; j0 < K; j0 += 8) {
-    uint4 v[8];
+  for (int j0 = 0; j0 < k_rt; j0 += kBatch) {
+    uint4 v[kBatch];
+    float w[kBatch];
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj)
-      if (j0 + jj < K) v[jj] = y[(size_t)s_slot[j0 + jj] * nvec + c];
+    for (int jj = 0; jj < kBatch; ++jj)
+      if (j0 + jj < k_rt) {
+        const int src = entry_lane<MODE>(en, j0 + jj);
+        const int slot = __builtin_amdgcn_readlane(en.slot, src);
+        w[jj] = lane_read(en.w, src);
+        if (r.active) v[jj] = load_row<STREAM>(y + (size_t)slot * nvec + r.c);
+      }
+    if (r.active) {
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj)
-      if (j0 + jj < K) accumulate8<E, MODE>(acc, v[jj], s_w[j0 + jj]);
+      for (int jj = 0; jj < kBatch; ++jj)
+        if (j0 + jj < k_rt) accumulate8<E, MODE>(acc, v[jj], w[jj]);
+    }
   }
-  out[(size_t)t * nvec + c] = make_uint4(E::pack(acc[0], acc[1]), E::pack(acc[2], acc[3]),
-                                         E::pack(acc[4], acc[5]), E::pack(acc[6], acc[7]));
+  if (r.active) store_row<STREAM>(out + (size_t)r.t * nvec + r.c, pack8<E>(acc));
 }
 
 // stub folded into the combine, 16-bit dispatched rows
-template <class In, class Out, int MODE>
-__global__ __launch_bounds__(kRowThreads) void stub_combine_rows_kernel(
+template <class In, class Out, int MODE, int KT, int STREAM>
+__global__ __launch_bounds__(kRowMaxThreads) void stub_combine_rows_kernel(
     const uint4* __restrict__ disp, const int32_t* __restrict__ indices, const float* __restrict__ weights,
     const int32_t* __restrict__ slot_of_entry, uint4* __restrict__ out, int stub_kind, int E, int E_l, int K,
-    int nvec, int nsplit) {
-  __shared__ int s_slot[MOE_A2A_MAX_TOPK];
-  __shared__ float s_w[MOE_A2A_MAX_TOPK];
-  __shared__ int s_k[MOE_A2A_MAX_TOPK];
-  __shared__ float s_f[MOE_A2A_MAX_TOPK];
-  const int t = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - t * nsplit;
-  order_entries(slot_of_entry, weights, t, K, MODE, s_slot, s_w, s_k);
-  if ((int)threadIdx.x < K)
-    s_f[threadIdx.x] = stub_factor(indices[(size_t)t * K + s_k[threadIdx.x]], stub_kind, E, E_l);
-  __syncthreads();
-  const int c = cs * kRowThreads + threadIdx.x;
-  if (c >= nvec) return;
+    int nvec, int per, int nsplit) {
+  constexpr int kBatch = KT > 0 ? KT : 4;
+  const int k_rt = KT ? KT : K;
+  const RowCut r = row_cut(nvec, per, nsplit);
+  EntryLanes en = load_entries<MODE>(slot_of_entry, weights, r.t, k_rt);
+  if (en.live)
+    en.f = stub_factor(indices[(size_t)r.t * k_rt + (threadIdx.x & (kWave - 1))], stub_kind, E, E_l);
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  for (int j0 = 0; j0 < K; j0 += 8) {
-    uint4 v[8];
+  for (int j0 = 0; j0 < k_rt; j0 += kBatch) {
+    uint4 v[kBatch];
+    float w[kBatch], f[kBatch];
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj)
-      if (j0 + jj < K) v[jj] = disp[(size_t)s_slot[j0 + jj] * nvec + c];
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-      if (j0 + jj >= K) continue;
-      const float s = s_f[j0 + jj];
-      uint32_t d[4];
-      unpack8(v[jj], d);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float a = In::lo(d[j]), b = In::hi(d[j]);
-        round_pair<Out>(a, b);
-        d[j] = Out::pack(a * s, b * s);
+    for (int jj = 0; jj < kBatch; ++jj)
+      if (j0 + jj < k_rt) {
+        const int src = entry_lane<MODE>(en, j0 + jj);
+        const int slot = __builtin_amdgcn_readlane(en.slot, src);
+        w[jj] = lane_read(en.w, src);
+        f[jj] = lane_read(en.f, src);
+        if (r.active) v[jj] = load_row<STREAM>(disp + (size_t)slot * nvec + r.c);
       }
-      accumulate8<Out, MODE>(acc, make_uint4(d[0], d[1], d[2], d[3]), s_w[j0 + jj]);
+    if (r.active) {
+#pragma unroll
+      for (int jj = 0; jj < kBatch; ++jj)
+        if (j0 + jj < k_rt) accumulate8<Out, MODE>(acc, stub_vec<In, Out>(v[jj], f[jj]), w[jj]);
     }
   }
-  out[(size_t)t * nvec + c] = make_uint4(Out::pack(acc[0], acc[1]), Out::pack(acc[2], acc[3]),
-                                         Out::pack(acc[4], acc[5]), Out::pack(acc[6], acc[7]));
+  if (r.active) store_row<STREAM>(out + (size_t)r.t * nvec + r.c, pack8<Out>(acc));
 }
 
 // stub folded into the combine, fp8 dispatched rows (16 columns per lane)
-template <class Out, int MODE>
-__global__ __launch_bounds__(kRowThreads) void stub_combine_fp8_kernel(
+template <class Out, int MODE, int KT, int STREAM>
+__global__ __launch_bounds__(kRowMaxThreads) void stub_combine_fp8_kernel(
     const uint4* __restrict__ disp_q, const float* __restrict__ disp_scale, const int32_t* __restrict__ indices,
     const float* __restrict__ weights, const int32_t* __restrict__ slot_of_entry, uint4* __restrict__ out,
-    int stub_kind, int E, int E_l, int K, int nblk, int nsplit) {
-  __shared__ int s_slot[MOE_A2A_MAX_TOPK];
-  __shared__ float s_w[MOE_A2A_MAX_TOPK];
-  __shared__ int s_k[MOE_A2A_MAX_TOPK];
-  __shared__ float s_f[MOE_A2A_MAX_TOPK];
-  const int t = blockIdx.x / nsplit;
-  const int cs = blockIdx.x - t * nsplit;
-  order_entries(slot_of_entry, weights, t, K, MODE, s_slot, s_w, s_k);
-  if ((int)threadIdx.x < K)
-    s_f[threadIdx.x] = stub_factor(indices[(size_t)t * K + s_k[threadIdx.x]], stub_kind, E, E_l);
-  __syncthreads();
-  const int c = cs * kRowThreads + threadIdx.x;
-  if (c >= nblk * 8) return;
+    int stub_kind, int E, int E_l, int K, int nblk, int per, int nsplit) {
+  constexpr int kBatch = KT > 0 ? KT : 4;
+  const int k_rt = KT ? KT : K;
+  const RowCut r = row_cut(nblk * 8, per, nsplit);
+  EntryLanes en = load_entries<MODE>(slot_of_entry, weights, r.t, k_rt);
+  if (en.live)
+    en.f = stub_factor(indices[(size_t)r.t * k_rt + (threadIdx.x & (kWave - 1))], stub_kind, E, E_l);
   float acc0[8], acc1[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc0[j] = acc1[j] = 0.f;
-  for (int j0 = 0; j0 < K; j0 += 4) {
-    uint4 v[4];
-    float sc[4];
+  for (int j0 = 0; j0 < k_rt; j0 += kBatch) {
+    uint4 v[kBatch];
+    float sc[kBatch], w[kBatch], f[kBatch];
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj)
-      if (j0 + jj < K) {
-        size_t row = (size_t)s_slot[j0 + jj];
-        v[jj] = disp_q[row * nblk * 8 + c];
-        sc[jj] = disp_scale[row * nblk + (c >> 3)];
+    for (int jj = 0; jj < kBatch; ++jj)
+      if (j0 + jj < k_rt) {
+        const int src = entry_lane<MODE>(en, j0 + jj);
+        const size_t row = (size_t)__builtin_amdgcn_readlane(en.slot, src);
+        w[jj] = lane_read(en.w, src);
+        f[jj] = lane_read(en.f, src);
+        if (r.active) {
+          v[jj] = load_row<STREAM>(disp_q + row * nblk * 8 + r.c);
+          sc[jj] = disp_scale[row * nblk + (r.c >> 3)];
+        }
       }
+    if (r.active) {
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      if (j0 + jj >= K) continue;
-      const float s = s_f[j0 + jj];
-      const uint32_t qw[4] = {v[jj].x, v[jj].y, v[jj].z, v[jj].w};
-      uint32_t o[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float f[4];
-        fp8x4_to_f32(qw[j], f);
-        o[2 * j] = Out::pack((f[0] * sc[jj]) * s, (f[1] * sc[jj]) * s);
-        o[2 * j + 1] = Out::pack((f[2] * sc[jj]) * s, (f[3] * sc[jj]) * s);
+      for (int jj = 0; jj < kBatch; ++jj) {
+        if (j0 + jj >= k_rt) continue;
+        uint4 o0, o1;
+        stub_vec_fp8<Out>(v[jj], sc[jj], f[jj], o0, o1);
+        accumulate8<Out, MODE>(acc0, o0, w[jj]);
+        accumulate8<Out, MODE>(acc1, o1, w[jj]);
       }
-      accumulate8<Out, MODE>(acc0, make_uint4(o[0], o[1], o[2], o[3]), s_w[j0 + jj]);
-      accumulate8<Out, MODE>(acc1, make_uint4(o[4], o[5], o[6], o[7]), s_w[j0 + jj]);
     }
   }
-  uint4* dst = out + ((size_t)t * nblk * 8 + c) * 2;
-  dst[0] = make_uint4(Out::pack(acc0[0], acc0[1]), Out::pack(acc0[2], acc0[3]), Out::pack(acc0[4], acc0[5]),
-                      Out::pack(acc0[6], acc0[7]));
-  dst[1] = make_uint4(Out::pack(acc1[0], acc1[1]), Out::pack(acc1[2], acc1[3]), Out::pack(acc1[4], acc1[5]),
-                      Out::pack(acc1[6], acc1[7]));
+  if (r.active) {
+    uint4* dst = out + ((size_t)r.t * nblk * 8 + r.c) * 2;
+    store_row<STREAM>(dst, pack8<Out>(acc0));
+    store_row<STREAM>(dst + 1, pack8<Out>(acc1));
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -833,12 +925,17 @@ int id_bits(int E) {
   return b;
 }
 
-// vectors per thread for the row kernels: fewer when the grid would otherwise be small
-int pick_unroll(int rows, int nvec) {
-  for (int u = 4; u > 1; u >>= 1) {
-    if (nvec >= kRowThreads * u && (long long)rows * ceil_div(nvec, kRowThreads * u) >= 2048) return u;
-  }
-  return 1;
+// column split of a row of nvec lanes; `unit` lanes must stay in one workgroup
+struct RowGeom {
+  int per, nsplit, threads;
+};
+RowGeom row_geom(int nvec, int unit = 1, int max_threads = kRowMaxThreads, int min_threads = kWave) {
+  RowGeom g;
+  g.nsplit = ceil_div(nvec, max_threads);
+  g.per = ceil_div(ceil_div(nvec, g.nsplit), unit) * unit;
+  g.threads = ceil_div(g.per, kWave) * kWave;
+  if (g.threads < min_threads) g.threads = min_threads;  // extra lanes only help with index work
+  return g;
 }
 
 template <typename F>
@@ -872,7 +969,7 @@ const char* moe_a2a_strerror(int code) {
 size_t moe_a2a_workspace_bytes(int T, int K, int E) {
   if (T < 0 || K < 1 || E < 1) return 0;
   long long R = (long long)T * K;
-  if (R <= kRouteSingleMaxRows) return 256;
+  if (R <= kRouteTilesMaxRows) return 256;
   long long ntiles = (R + kRouteThreads - 1) / kRouteThreads;
   return align_up((size_t)ntiles * (size_t)E * sizeof(int32_t), 256);
 }
@@ -888,24 +985,24 @@ int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_ran
               src_of_slot, meta, status};
   const size_t lds_w = (size_t)kRouteWaves * E * sizeof(int);
   const size_t lds_starts = (size_t)(W + 1) * sizeof(int);
-  if (a.R <= kRouteSingleMaxRows) {
-    size_t lds = lds_w + (size_t)E * sizeof(int) + (kRouteWaves + 1) * sizeof(int) + lds_starts;
-    set_max_lds(route_single_kernel, lds);
-    return launch(KID_ROUTE_SINGLE, route_single_kernel, dim3(1), dim3(kRouteThreads), lds, stream, a);
+  if (a.R <= kRouteTilesMaxRows) {
+    size_t lds = lds_w + 2 * (size_t)E * sizeof(int) + (kRouteWaves + 1) * sizeof(int) + lds_starts;
+    set_max_lds(route_tiles_kernel, lds);
+    return launch(KID_ROUTE_TILES, route_tiles_kernel, dim3(a.R ? ceil_div(a.R, kRouteThreads) : 1),
+                  dim3(kRouteThreads), lds, stream, a);
   }
   if (!workspace || workspace_bytes < moe_a2a_workspace_bytes(T, K, E)) return MOE_A2A_E_WORKSPACE;
   int ntiles = ceil_div(a.R, kRouteThreads);
   int32_t* tile = (int32_t*)workspace;
   set_max_lds(route_hist_kernel, lds_w);
-  if (int rc = launch(KID_ROUTE_HIST, route_hist_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w, stream, a, tile,
-                      ntiles))
+  if (int rc = launch(KID_ROUTE_HIST, route_hist_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w, stream, a, tile))
     return rc;
-  if (int rc = launch(KID_ROUTE_SCAN, route_scan_kernel, dim3(1), dim3(kRouteThreads), 0, stream, tile, E * ntiles,
-                      E, ntiles, counts, offsets))
+  if (int rc = launch(KID_ROUTE_SCAN, route_scan_kernel, dim3(1), dim3(kRouteThreads), 0, stream, tile, E, ntiles,
+                      counts, offsets))
     return rc;
   set_max_lds(route_rank_kernel, lds_w + lds_starts);
   return launch(KID_ROUTE_RANK, route_rank_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w + lds_starts, stream, a,
-                (const int32_t*)tile, ntiles);
+                (const int32_t*)tile);
 }
 
 static int check_rows(const void* a, const void* b, int T, int K, int H, int mult) {
@@ -916,26 +1013,39 @@ static int check_rows(const void* a, const void* b, int T, int K, int H, int mul
   return 0;
 }
 
+// bytes a row kernel moves decide its cache policy (see load_row / store_row)
+#ifndef MOE_A2A_STREAM_BYTES
+#define MOE_A2A_STREAM_BYTES (192ll << 20)
+#endif
+static bool streams(long long rows_in, long long rows_out, int H, int in_bytes, int out_bytes) {
+  return (rows_in * in_bytes + rows_out * out_bytes) * (long long)H > MOE_A2A_STREAM_BYTES;
+}
+
 int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, int T, int K, int H,
                      moe_a2a_stream_t stream_) {
   if (int rc = check_rows(x, disp_x, T, K, H, 8)) return rc;
   if (T == 0) return 0;
   if (!slot_of_entry) return MOE_A2A_E_NULL;
-  hipStream_t stream = (hipStream_t)stream_;
   const int nvec = H / 8;
-  const int U = pick_unroll(T, nvec);
-  const int nsplit = ceil_div(nvec, kRowThreads * U);
-  dim3 grid((unsigned)T * nsplit), block(kRowThreads);
-  const uint4* xs = (const uint4*)x;
-  uint4* ds = (uint4*)disp_x;
-  switch (U) {
-    case 4: return launch(KID_DISPATCH, dispatch_rows_kernel<4>, grid, block, 0, stream, xs, slot_of_entry, ds, K, nvec, nsplit);
-    case 2: return launch(KID_DISPATCH, dispatch_rows_kernel<2>, grid, block, 0, stream, xs, slot_of_entry, ds, K, nvec, nsplit);
-    default: return launch(KID_DISPATCH, dispatch_rows_kernel<1>, grid, block, 0, stream, xs, slot_of_entry, ds, K, nvec, nsplit);
-  }
+  const RowGeom g = row_geom(nvec);
+  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
+  if (streams(T, (long long)T * K, H, 2, 2))
+    return launch(KID_DISPATCH, dispatch_rows_kernel<1>, grid, block, 0, (hipStream_t)stream_, (const uint4*)x,
+                  slot_of_entry, (uint4*)disp_x, K, nvec, g.per, g.nsplit);
+  return launch(KID_DISPATCH, dispatch_rows_kernel<0>, grid, block, 0, (hipStream_t)stream_, (const uint4*)x,
+                slot_of_entry, (uint4*)disp_x, K, nvec, g.per, g.nsplit);
 }
 
 int moe_a2a_fused_max_rows(void) { return kFusedMaxRows; }
+
+int moe_a2a_fused_ok(int T, int K, int H) {
+  if (T < 1 || K < 1 || H < 8) return 0;
+  const long long R = (long long)T * K;
+  if (R > kFusedMaxRows) return 0;
+  const RowGeom g = row_geom(H / 8, 1, kFusedMaxThreads, 256);
+  // every workgroup reads the whole routing table: keep that traffic far below the payload
+  return R * T * g.nsplit <= kFusedMaxTableReads ? 1 : 0;
+}
 
 int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
                            int K, int E, int W, int H, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
@@ -946,20 +1056,12 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
   if (int rc = check_rows(x, disp_x, T, K, H, 8)) return rc;
   if (!counts || !offsets) return MOE_A2A_E_NULL;
   if (T > 0 && (!indices || !slot_of_entry || !src_of_slot || !meta)) return MOE_A2A_E_NULL;
-  hipStream_t stream = (hipStream_t)stream_;
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), counts, offsets, slot_of_entry,
               src_of_slot, meta, status};
   const int nvec = H / 8;
-  const int U = pick_unroll(T, nvec);
-  const int nsplit = ceil_div(nvec, kRowThreads * U);
-  dim3 grid((unsigned)T * nsplit + 1), block(kRowThreads);
-  const uint4* xs = (const uint4*)x;
-  uint4* ds = (uint4*)disp_x;
-  switch (U) {
-    case 4: return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<4>, grid, block, 0, stream, a, xs, ds, nvec, nsplit);
-    case 2: return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<2>, grid, block, 0, stream, a, xs, ds, nvec, nsplit);
-    default: return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<1>, grid, block, 0, stream, a, xs, ds, nvec, nsplit);
-  }
+  const RowGeom g = row_geom(nvec, 1, kFusedMaxThreads, 256);
+  return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel, dim3((unsigned)T * g.nsplit + 1), dim3(g.threads), 0,
+                (hipStream_t)stream_, a, (const uint4*)x, (uint4*)disp_x, nvec, g.per, g.nsplit);
 }
 
 int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry, uint8_t* disp_q,
@@ -970,13 +1072,19 @@ int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry
   if (!slot_of_entry || !disp_scale) return MOE_A2A_E_NULL;
   hipStream_t stream = (hipStream_t)stream_;
   const int nblk = H / MOE_A2A_FP8_BLOCK;
-  const int nsplit = ceil_div(nblk, kRowThreads / 8);
-  dim3 grid((unsigned)T * nsplit), block(kRowThreads);
-  if (x_type == MOE_A2A_BF16)
-    return launch(KID_DISPATCH_FP8, dispatch_fp8_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x, slot_of_entry,
-                  (uint4*)disp_q, disp_scale, K, nblk, nsplit);
-  return launch(KID_DISPATCH_FP8, dispatch_fp8_kernel<F16>, grid, block, 0, stream, (const uint4*)x, slot_of_entry,
-                (uint4*)disp_q, disp_scale, K, nblk, nsplit);
+  const RowGeom g = row_geom(nblk * 8, 8);
+  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
+  const bool st = streams(T, (long long)T * K, H, 2, 1);
+#define FP8_LAUNCH(EL, ST)                                                                                       \
+  return launch(KID_DISPATCH_FP8, dispatch_fp8_kernel<EL, ST>, grid, block, 0, stream, (const uint4*)x, slot_of_entry, \
+                (uint4*)disp_q, disp_scale, K, nblk, g.per, g.nsplit)
+  if (x_type == MOE_A2A_BF16) {
+    if (st) FP8_LAUNCH(Bf16, 1);
+    FP8_LAUNCH(Bf16, 0);
+  }
+  if (st) FP8_LAUNCH(F16, 1);
+  FP8_LAUNCH(F16, 0);
+#undef FP8_LAUNCH
 }
 
 static bool known_type(int t) { return t == MOE_A2A_F16 || t == MOE_A2A_BF16; }
@@ -991,34 +1099,49 @@ int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta,
   if (!meta) return MOE_A2A_E_NULL;
   hipStream_t stream = (hipStream_t)stream_;
   const int E_l = E / W;
-  dim3 block(kRowThreads);
+  const bool st = streams(R, R, H, disp_scale ? 1 : 2, 2);
   if (disp_scale) {
-    const int nblk = H / MOE_A2A_FP8_BLOCK;
-    const int nsplit = ceil_div(nblk * 8, kRowThreads);
-    dim3 grid((unsigned)R * nsplit);
-    if (out_type == MOE_A2A_BF16)
-      return launch(KID_STUB_FP8, stub_fp8_kernel<Bf16>, grid, block, 0, stream, (const uint4*)disp, disp_scale, meta,
-                    (uint4*)y, stub_kind, E, E_l, nblk, nsplit);
-    return launch(KID_STUB_FP8, stub_fp8_kernel<F16>, grid, block, 0, stream, (const uint4*)disp, disp_scale, meta,
-                  (uint4*)y, stub_kind, E, E_l, nblk, nsplit);
+    const int nvec = H / 8;
+    const RowGeom g = row_geom(nvec);
+    dim3 grid((unsigned)R * g.nsplit), block(g.threads);
+#define STUB8_LAUNCH(OUT, ST)                                                                                   \
+  return launch(KID_STUB_FP8, stub_fp8_kernel<OUT, ST>, grid, block, 0, stream, (const uint2*)disp, disp_scale, meta, \
+                (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit)
+    if (out_type == MOE_A2A_BF16) {
+      if (st) STUB8_LAUNCH(Bf16, 1);
+      STUB8_LAUNCH(Bf16, 0);
+    }
+    if (st) STUB8_LAUNCH(F16, 1);
+    STUB8_LAUNCH(F16, 0);
+#undef STUB8_LAUNCH
   }
   const int nvec = H / 8;
-  const int U = pick_unroll(R, nvec) >= 2 ? 2 : 1;
-  const int nsplit = ceil_div(nvec, kRowThreads * U);
-  dim3 grid((unsigned)R * nsplit);
-#define STUB_LAUNCH(IN, OUT, UU)                                                                              \
-  return launch(KID_STUB, stub_rows_kernel<IN, OUT, UU>, grid, block, 0, stream, (const uint4*)disp, meta, \
-                (uint4*)y, stub_kind, E, E_l, nvec, nsplit)
-#define STUB_TYPES(UU)                                                     \
-  if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_BF16) STUB_LAUNCH(Bf16, Bf16, UU); \
-  if (in_type == MOE_A2A_F16 && out_type == MOE_A2A_F16) STUB_LAUNCH(F16, F16, UU);     \
-  if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_F16) STUB_LAUNCH(Bf16, F16, UU);   \
-  STUB_LAUNCH(F16, Bf16, UU)
-  if (U == 2) { STUB_TYPES(2); }
-  STUB_TYPES(1);
-#undef STUB_TYPES
+  const RowGeom g = row_geom(nvec);
+  dim3 grid((unsigned)R * g.nsplit), block(g.threads);
+#define STUB_LAUNCH(IN, OUT)                                                                                  \
+  {                                                                                                           \
+    if (st)                                                                                                   \
+      return launch(KID_STUB, stub_rows_kernel<IN, OUT, 1>, grid, block, 0, stream, (const uint4*)disp, meta, \
+                    (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit);                                     \
+    return launch(KID_STUB, stub_rows_kernel<IN, OUT, 0>, grid, block, 0, stream, (const uint4*)disp, meta,   \
+                  (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit);                                       \
+  }
+  if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_BF16) STUB_LAUNCH(Bf16, Bf16)
+  if (in_type == MOE_A2A_F16 && out_type == MOE_A2A_F16) STUB_LAUNCH(F16, F16)
+  if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_F16) STUB_LAUNCH(Bf16, F16)
+  STUB_LAUNCH(F16, Bf16)
 #undef STUB_LAUNCH
 }
+
+// top-k values with a specialised kernel; any other K takes the generic one (KT = 0)
+#define MOE_A2A_SWITCH_KT(K, CALL) \
+  switch (K) {                     \
+    case 2: CALL(2);               \
+    case 4: CALL(4);               \
+    case 6: CALL(6);               \
+    case 8: CALL(8);               \
+    default: CALL(0);              \
+  }
 
 int moe_a2a_combine(const void* expert_y, const float* weights, const int32_t* slot_of_entry, int mode,
                     int elem_type, void* out, int T, int K, int H, moe_a2a_stream_t stream_) {
@@ -1029,17 +1152,32 @@ int moe_a2a_combine(const void* expert_y, const float* weights, const int32_t* s
   if (!weights || !slot_of_entry) return MOE_A2A_E_NULL;
   hipStream_t stream = (hipStream_t)stream_;
   const int nvec = H / 8;
-  const int nsplit = ceil_div(nvec, kRowThreads);
-  dim3 grid((unsigned)T * nsplit), block(kRowThreads);
-#define COMBINE_LAUNCH(EL, MD)                                                                                  \
-  return launch(KID_COMBINE, combine_rows_kernel<EL, MD>, grid, block, 0, stream, (const uint4*)expert_y, weights, \
-                slot_of_entry, (uint4*)out, K, nvec, nsplit)
-  if (elem_type == MOE_A2A_BF16) {
-    if (mode == MOE_A2A_COMBINE_STRICT) COMBINE_LAUNCH(Bf16, MOE_A2A_COMBINE_STRICT);
-    COMBINE_LAUNCH(Bf16, MOE_A2A_COMBINE_F32);
+  const RowGeom g = row_geom(nvec);
+  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
+  const bool st = streams((long long)T * K, T, H, 2, 2);
+#define COMBINE_LAUNCH(EL, MD, KT)                                                                            \
+  {                                                                                                           \
+    if (st)                                                                                                   \
+      return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 1>, grid, block, 0, stream,                  \
+                    (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit);   \
+    return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 0>, grid, block, 0, stream,                    \
+                  (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit);     \
   }
-  if (mode == MOE_A2A_COMBINE_STRICT) COMBINE_LAUNCH(F16, MOE_A2A_COMBINE_STRICT);
-  COMBINE_LAUNCH(F16, MOE_A2A_COMBINE_F32);
+#define CALL_BS(KT) COMBINE_LAUNCH(Bf16, MOE_A2A_COMBINE_STRICT, KT)
+#define CALL_BF(KT) COMBINE_LAUNCH(Bf16, MOE_A2A_COMBINE_F32, KT)
+#define CALL_HS(KT) COMBINE_LAUNCH(F16, MOE_A2A_COMBINE_STRICT, KT)
+#define CALL_HF(KT) COMBINE_LAUNCH(F16, MOE_A2A_COMBINE_F32, KT)
+  const bool strict = mode == MOE_A2A_COMBINE_STRICT;
+  if (elem_type == MOE_A2A_BF16) {
+    if (strict) MOE_A2A_SWITCH_KT(K, CALL_BS)
+    MOE_A2A_SWITCH_KT(K, CALL_BF)
+  }
+  if (strict) MOE_A2A_SWITCH_KT(K, CALL_HS)
+  MOE_A2A_SWITCH_KT(K, CALL_HF)
+#undef CALL_BS
+#undef CALL_BF
+#undef CALL_HS
+#undef CALL_HF
 #undef COMBINE_LAUNCH
 }
 
@@ -1055,41 +1193,77 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
   if (!indices || !weights || !slot_of_entry) return MOE_A2A_E_NULL;
   hipStream_t stream = (hipStream_t)stream_;
   const int E_l = E / W;
-  dim3 block(kRowThreads);
   const bool strict = mode == MOE_A2A_COMBINE_STRICT;
+  const bool st = streams((long long)T * K, T, H, disp_scale ? 1 : 2, 2);
   if (disp_scale) {
     const int nblk = H / MOE_A2A_FP8_BLOCK;
-    const int nsplit = ceil_div(nblk * 8, kRowThreads);
-    dim3 grid((unsigned)T * nsplit);
-#define SC8_LAUNCH(OUT, MD)                                                                                   \
-  return launch(KID_STUB_COMBINE, stub_combine_fp8_kernel<OUT, MD>, grid, block, 0, stream, (const uint4*)disp, \
-                disp_scale, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K, nblk, nsplit)
+    const RowGeom g = row_geom(nblk * 8);
+    dim3 grid((unsigned)T * g.nsplit), block(g.threads);
+#define SC8_LAUNCH(OUT, MD, KT)                                                                                 \
+  {                                                                                                             \
+    if (st)                                                                                                     \
+      return launch(KID_STUB_COMBINE, stub_combine_fp8_kernel<OUT, MD, KT, 1>, grid, block, 0, stream,          \
+                    (const uint4*)disp, disp_scale, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, \
+                    E_l, K, nblk, g.per, g.nsplit);                                                             \
+    return launch(KID_STUB_COMBINE, stub_combine_fp8_kernel<OUT, MD, KT, 0>, grid, block, 0, stream,            \
+                  (const uint4*)disp, disp_scale, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E,   \
+                  E_l, K, nblk, g.per, g.nsplit);                                                               \
+  }
+#define CALL_BS(KT) SC8_LAUNCH(Bf16, MOE_A2A_COMBINE_STRICT, KT)
+#define CALL_BF(KT) SC8_LAUNCH(Bf16, MOE_A2A_COMBINE_F32, KT)
+#define CALL_HS(KT) SC8_LAUNCH(F16, MOE_A2A_COMBINE_STRICT, KT)
+#define CALL_HF(KT) SC8_LAUNCH(F16, MOE_A2A_COMBINE_F32, KT)
     if (out_type == MOE_A2A_BF16) {
-      if (strict) SC8_LAUNCH(Bf16, MOE_A2A_COMBINE_STRICT);
-      SC8_LAUNCH(Bf16, MOE_A2A_COMBINE_F32);
+      if (strict) MOE_A2A_SWITCH_KT(K, CALL_BS)
+      MOE_A2A_SWITCH_KT(K, CALL_BF)
     }
-    if (strict) SC8_LAUNCH(F16, MOE_A2A_COMBINE_STRICT);
-    SC8_LAUNCH(F16, MOE_A2A_COMBINE_F32);
+    if (strict) MOE_A2A_SWITCH_KT(K, CALL_HS)
+    MOE_A2A_SWITCH_KT(K, CALL_HF)
+#undef CALL_BS
+#undef CALL_BF
+#undef CALL_HS
+#undef CALL_HF
 #undef SC8_LAUNCH
   }
   const int nvec = H / 8;
-  const int nsplit = ceil_div(nvec, kRowThreads);
-  dim3 grid((unsigned)T * nsplit);
-#define SC_LAUNCH(IN, OUT, MD)                                                                                     \
-  return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD>, grid, block, 0, stream, (const uint4*)disp, \
-                indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K, nvec, nsplit)
-#define SC_MODES(IN, OUT)                                  \
-  {                                                        \
-    if (strict) SC_LAUNCH(IN, OUT, MOE_A2A_COMBINE_STRICT); \
-    SC_LAUNCH(IN, OUT, MOE_A2A_COMBINE_F32);               \
+  const RowGeom g = row_geom(nvec);
+  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
+#define SC_LAUNCH(IN, OUT, MD, KT)                                                                              \
+  {                                                                                                             \
+    if (st)                                                                                                     \
+      return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD, KT, 1>, grid, block, 0, stream,     \
+                    (const uint4*)disp, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K,     \
+                    nvec, g.per, g.nsplit);                                                                     \
+    return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD, KT, 0>, grid, block, 0, stream,       \
+                  (const uint4*)disp, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K, nvec, \
+                  g.per, g.nsplit);                                                                             \
   }
-  if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_BF16) SC_MODES(Bf16, Bf16)
-  if (in_type == MOE_A2A_F16 && out_type == MOE_A2A_F16) SC_MODES(F16, F16)
-  if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_F16) SC_MODES(Bf16, F16)
-  SC_MODES(F16, Bf16)
-#undef SC_MODES
+#define CALL_BS(KT) SC_LAUNCH(Bf16, Bf16, MOE_A2A_COMBINE_STRICT, KT)
+#define CALL_BF(KT) SC_LAUNCH(Bf16, Bf16, MOE_A2A_COMBINE_F32, KT)
+#define CALL_HS(KT) SC_LAUNCH(F16, F16, MOE_A2A_COMBINE_STRICT, KT)
+#define CALL_HF(KT) SC_LAUNCH(F16, F16, MOE_A2A_COMBINE_F32, KT)
+  if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_BF16) {
+    if (strict) MOE_A2A_SWITCH_KT(K, CALL_BS)
+    MOE_A2A_SWITCH_KT(K, CALL_BF)
+  }
+  if (in_type == MOE_A2A_F16 && out_type == MOE_A2A_F16) {
+    if (strict) MOE_A2A_SWITCH_KT(K, CALL_HS)
+    MOE_A2A_SWITCH_KT(K, CALL_HF)
+  }
+  // mixed element types: generic kernel only
+  if (in_type == MOE_A2A_BF16) {
+    if (strict) SC_LAUNCH(Bf16, F16, MOE_A2A_COMBINE_STRICT, 0)
+    SC_LAUNCH(Bf16, F16, MOE_A2A_COMBINE_F32, 0)
+  }
+  if (strict) SC_LAUNCH(F16, Bf16, MOE_A2A_COMBINE_STRICT, 0)
+  SC_LAUNCH(F16, Bf16, MOE_A2A_COMBINE_F32, 0)
+#undef CALL_BS
+#undef CALL_BF
+#undef CALL_HS
+#undef CALL_HF
 #undef SC_LAUNCH
 }
+#undef MOE_A2A_SWITCH_KT
 
 int moe_a2a_timer_begin(int capacity) {
   if (g_timer.active || capacity < 1) return MOE_A2A_E_STATE;

@@ -58,7 +58,7 @@ def compare(cfg, world, dev, stub_kind, combine_mode=0, fp8=False, fuse_route=Tr
 
 
 @pytest.mark.parametrize("name", GOLDEN_CASES)
-@pytest.mark.parametrize("fuse_route", [True, False])
+@pytest.mark.parametrize("fuse_route", ["always", False])
 def test_reference_vectors(gpu_device, name, fuse_route):
     """Against the outputs the reference's own PyTorchAllToAll wrote (tests/golden/)."""
     cfg, world, expected = load_golden(name)
@@ -84,7 +84,7 @@ def test_reference_vectors(gpu_device, name, fuse_route):
 def test_reference_specs_whole_world(gpu_device, spec, dtype):
     """The reference's 9 test specs (all2all/task.yml:59-68), all 8 ranks resident at once."""
     cfg, world = C.generate_world(**spec, dtype=dtype)
-    for fuse in (True, False):
+    for fuse in ("always", True, False):
         compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=fuse)
 
 
@@ -92,7 +92,7 @@ def test_reference_specs_whole_world(gpu_device, spec, dtype):
 @pytest.mark.parametrize("mode", [C.COMBINE_STRICT, C.COMBINE_F32], ids=["strict", "f32"])
 def test_named_workloads(gpu_device, name, scale, mode):
     wl = C.generate_workload(name, tokens_scale=scale)
-    for fuse in (True, False):
+    for fuse in ("always", True, False):
         o, d = compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, combine_mode=mode, fuse_route=fuse)
     if name == "skew_world":
         assert int(o["counts"].max()) <= wl.total_tokens  # one row per token and expert at most
@@ -110,6 +110,18 @@ def test_multi_workgroup_routing(gpu_device):
     compare(cfg, world, gpu_device, C.STUB_EXPERT_FRACTION)
 
 
+def test_huge_routing_table(gpu_device):
+    """R = 264000 routed rows: more tiles than the rank kernel sums by itself, so the
+    column-scan kernel runs too."""
+    g = torch.Generator().manual_seed(9)
+    T, K, E, H = 33000, 8, 32, 64
+    cfg = C.MoEConfig(E, K, H, T + 1, torch.float16, torch.float16)
+    idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    world = [C.RankData(T, idx, torch.rand(T, K, generator=g), torch.randn(T, H, generator=g).to(torch.float16))]
+    world += [C.RankData.empty(cfg) for _ in range(7)]
+    compare(cfg, world, gpu_device, C.STUB_OWNER_RANK)
+
+
 def test_fp8_dispatch(gpu_device):
     wl = C.generate_workload("fp8_dispatch", tokens_scale=512 / 4096)
     compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, fp8=True)
@@ -124,8 +136,22 @@ def test_duplicate_experts_and_ragged_world(gpu_device):
     for n in [3, 0, 8, 1]:
         world.append(C.RankData(n, torch.randint(0, 16, (n, 4), generator=g).to(torch.int32),
                                 torch.rand(n, 4, generator=g), torch.randn(n, 2880, generator=g).to(torch.bfloat16)))
-    for fuse in (True, False):
+    for fuse in ("always", True, False):
         compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=fuse)
+
+
+@pytest.mark.parametrize("E,K,T,H", [(1024, 3, 300, 128), (64, 32, 40, 256), (8, 1, 17, 64), (48, 5, 700, 1032)])
+def test_limits_and_generic_topk(gpu_device, E, K, T, H):
+    """Largest expert count (LDS beyond 64 KB), largest top-k, K without a specialised kernel,
+    H that is not a multiple of 64 lanes."""
+    g = torch.Generator().manual_seed(E + K)
+    cfg = C.MoEConfig(E, K, H, T + 1, torch.bfloat16, torch.bfloat16)
+    idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    world = [C.RankData.empty(cfg) for _ in range(8)]
+    world[3] = C.RankData(T, idx, torch.rand(T, K, generator=g), torch.randn(T, H, generator=g).to(torch.bfloat16))
+    for fuse in ("always", False):
+        for mode in (C.COMBINE_STRICT, C.COMBINE_F32):
+            compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, combine_mode=mode, fuse_route=fuse)
 
 
 def test_custom_kernel_contract(gpu_device):
