@@ -46,7 +46,7 @@ def parse_args():
     p.add_argument("--fuse-stub", action="store_true", help="fold the expert stub into the combine")
     p.add_argument("--bf16-dispatch", action="store_true", help="fp8 workload with a 16-bit dispatch")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    p.add_argument("--no-cold", action="store_true", help="skip the cold-cache leg")
+    p.add_argument("--cold", action="store_true", help="add a leg with caches flushed before every step")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
     return p.parse_args()
 
@@ -183,7 +183,7 @@ def main():
         roofline=roofline,
     )
 
-    if not args.no_cold:
+    if args.cold:
         # cold caches: overwrite 1 GiB (4x the 256 MB Infinity Cache) before every step
         flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         n_cold = min(args.steps, 30)

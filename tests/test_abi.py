@@ -1,0 +1,122 @@
+"""The C-ABI library on a machine without a GPU: it loads, exports every symbol the header
+declares, and rejects bad arguments on the host before any launch."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from kernel_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "moe_a2a.h")
+
+E_NULL, E_SHAPE, E_DTYPE, E_WORKSPACE, E_ALIGN, E_STATE = -1, -2, -3, -4, -5, -6
+A = 0x1000  # any non-NULL, 16-byte aligned address; never dereferenced on the host
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(moe_a2a_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == sorted(_lib.PROTOTYPES)
+
+
+def test_every_declared_symbol_is_exported():
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(raw, name), f"{name} is declared in include/moe_a2a.h but not exported"
+
+
+def test_version_strings_and_queries(lib):
+    assert lib.moe_a2a_abi_version() == _lib.ABI_VERSION
+    assert lib.moe_a2a_strerror(0) == b"success"
+    for code in (E_NULL, E_SHAPE, E_DTYPE, E_WORKSPACE, E_ALIGN, E_STATE):
+        assert lib.moe_a2a_strerror(code).startswith(b"moe_a2a:")
+    assert lib.moe_a2a_kernel_name(-1) == b"unknown"
+    names = set()
+    k = 0
+    while lib.moe_a2a_kernel_name(k) != b"unknown":
+        names.add(lib.moe_a2a_kernel_name(k))
+        k += 1
+    assert {b"route_tiles", b"route_dispatch", b"dispatch_rows", b"dispatch_fp8", b"combine_rows"} <= names
+    # small tables route in one launch and need only the minimum scratch
+    assert lib.moe_a2a_workspace_bytes(256, 8, 256) == 256
+    assert lib.moe_a2a_workspace_bytes(16384, 4, 128) >= 64 * 128 * 4
+    assert lib.moe_a2a_workspace_bytes(-1, 8, 256) == 0
+    assert lib.moe_a2a_fused_max_rows() >= 2048
+    assert lib.moe_a2a_fused_ok(256, 8, 7168) == 1  # the headline shape takes the one-launch path
+    assert lib.moe_a2a_fused_ok(16384, 4, 4096) == 0
+    assert lib.moe_a2a_fused_ok(1024, 6, 2048) == 0  # table re-reads would rival the payload
+
+
+def test_route_rejects_bad_arguments(lib):
+    def route(T=4, K=2, E=8, W=2, indices=A, counts=A, offsets=A, soe=A, sos=A, meta=A, ws=A, wsb=1 << 20):
+        return lib.moe_a2a_route(indices, None, 0, T, K, E, W, counts, offsets, soe, sos, meta, None, ws, wsb, None)
+
+    assert route(K=0) == E_SHAPE
+    assert route(K=33) == E_SHAPE
+    assert route(E=0) == E_SHAPE
+    assert route(E=1025) == E_SHAPE
+    assert route(E=9, W=2) == E_SHAPE  # experts must split evenly over ranks
+    assert route(W=0) == E_SHAPE
+    assert route(T=-1) == E_SHAPE
+    assert route(T=1 << 30, K=8) == E_SHAPE
+    assert route(counts=None) == E_NULL
+    assert route(indices=None) == E_NULL
+    assert route(meta=None) == E_NULL
+    # a table beyond the one-launch limit needs the workspace
+    assert route(T=40000, K=8, E=8, W=2, ws=None) == E_WORKSPACE
+    assert route(T=40000, K=8, E=8, W=2, wsb=16) == E_WORKSPACE
+
+
+def test_row_functions_reject_bad_arguments(lib):
+    assert lib.moe_a2a_dispatch(A, A, A, 4, 2, 12, None) == E_SHAPE  # H % 8
+    assert lib.moe_a2a_dispatch(A, A, A, 4, 0, 64, None) == E_SHAPE
+    assert lib.moe_a2a_dispatch(None, A, A, 4, 2, 64, None) == E_NULL
+    assert lib.moe_a2a_dispatch(A + 4, A, A, 4, 2, 64, None) == E_ALIGN
+    assert lib.moe_a2a_dispatch(A, None, A, 4, 2, 64, None) == E_NULL
+    assert lib.moe_a2a_dispatch(A, A, A, 0, 2, 64, None) == 0  # nothing to do, nothing launched
+    assert lib.moe_a2a_dispatch_fp8(A, 7, A, A, A, 4, 2, 128, None) == E_DTYPE
+    assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, A, 4, 2, 64, None) == E_SHAPE  # H % 128
+    assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, None, 4, 2, 128, None) == E_NULL
+    assert lib.moe_a2a_stub(A, None, A, 5, _lib.BF16, 0, 8, 2, A, 8, 64, None) == E_DTYPE
+    assert lib.moe_a2a_stub(A, None, A, _lib.BF16, _lib.BF16, 9, 8, 2, A, 8, 64, None) == E_DTYPE
+    assert lib.moe_a2a_stub(A, None, A, _lib.BF16, _lib.BF16, 0, 9, 2, A, 8, 64, None) == E_SHAPE
+    assert lib.moe_a2a_stub(A, None, None, _lib.BF16, _lib.BF16, 0, 8, 2, A, 8, 64, None) == E_NULL
+    assert lib.moe_a2a_combine(A, A, A, 3, _lib.BF16, A, 4, 2, 64, None) == E_DTYPE
+    assert lib.moe_a2a_combine(A, A, A, 0, 4, A, 4, 2, 64, None) == E_DTYPE
+    assert lib.moe_a2a_combine(A, None, A, 0, _lib.BF16, A, 4, 2, 64, None) == E_NULL
+    assert lib.moe_a2a_combine(A, A, A, 0, _lib.BF16, A + 8, 4, 2, 64, None) == E_ALIGN
+    assert lib.moe_a2a_stub_combine(A, None, None, A, A, 0, _lib.BF16, _lib.BF16, 0, 8, 2, A, 4, 2, 64, None) == E_NULL
+    assert lib.moe_a2a_stub_combine(A, None, A, A, A, 0, _lib.BF16, _lib.BF16, 0, 8, 3, A, 4, 2, 64, None) == E_SHAPE
+    big = lib.moe_a2a_fused_max_rows() // 8 + 1
+    assert lib.moe_a2a_route_dispatch(A, A, None, 0, big, 8, 8, 2, 64, A, A, A, A, A, None, A, None) == E_SHAPE
+
+
+def test_timer_needs_begin_first(lib):
+    ids = (ctypes.c_int * 4)()
+    us = (ctypes.c_float * 4)()
+    assert lib.moe_a2a_timer_end(ids, us, 4) == E_STATE
+    assert lib.moe_a2a_timer_begin(0) == E_STATE
+
+
+def test_error_wrapper_raises_with_message(lib):
+    with pytest.raises(_lib.MoeA2AError) as e:
+        _lib.check(E_ALIGN, "moe_a2a_dispatch")
+    assert "16-byte" in str(e.value) and e.value.code == E_ALIGN
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmoe_a2a.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()
