@@ -48,17 +48,24 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--cold", action="store_true", help="add a leg with caches flushed before every step")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
+    p.add_argument("--calibrate-copy", action="store_true",
+                   help="end with three plain 256 MiB device copies (a known-size reference for rocprof counters)")
     return p.parse_args()
 
 
-def kernel_times(lib, run, steps, torch):
-    """Per-kernel GPU durations (µs) of `steps` eager passes, from the library's launch timer."""
+def kernel_times(lib, run_n, steps, torch, before_each=None):
+    """Per-kernel GPU durations (µs) of `steps` passes launched back to back from C, from the
+    library's launch timer (HIP events bound to each launch)."""
     cap = steps * 8
     rc = lib.moe_a2a_timer_begin(cap)
     if rc != 0:
         raise RuntimeError(f"moe_a2a_timer_begin: {lib.moe_a2a_strerror(rc).decode()}")
-    for _ in range(steps):
-        run()
+    if before_each is None:
+        run_n(steps)
+    else:
+        for _ in range(steps):
+            before_each()
+            run_n(1)
     torch.cuda.synchronize()
     ids = (ctypes.c_int * cap)()
     us = (ctypes.c_float * cap)()
@@ -67,6 +74,33 @@ def kernel_times(lib, run, steps, torch):
     for i in range(n):
         per.setdefault(lib.moe_a2a_kernel_name(ids[i]).decode(), []).append(float(us[i]))
     return per
+
+
+class ForwardArgs(ctypes.Structure):
+    """Mirror of moe_a2a_forward_args in kernel_amd/csrc/bench_loop.cpp."""
+    _fields_ = ([(n, ctypes.c_void_p) for n in ("x", "indices", "weights", "rank_start")] +
+                [(n, ctypes.c_int) for n in ("src_rank", "T", "K", "E", "W", "H", "in_type", "out_type", "fp8_dispatch",
+                                             "stub_kind", "combine_mode", "fuse_route", "fuse_stub")] +
+                [(n, ctypes.c_void_p) for n in ("counts", "offsets", "slot_of_entry", "src_of_slot", "meta", "status",
+                                                "disp", "disp_scale", "expert_y", "out", "workspace")] +
+                [("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p)])
+
+
+def c_loop(step):
+    """run(n): n back-to-back steps launched from C with the planned step's own arguments."""
+    from kernel_amd import build as _build
+
+    loop = ctypes.CDLL(_build.BENCH_LIB_PATH)
+    loop.moe_a2a_bench_steps.restype = ctypes.c_int
+    loop.moe_a2a_bench_steps.argtypes = [ctypes.c_int, ctypes.POINTER(ForwardArgs), ctypes.POINTER(ForwardArgs)]
+    sets = [ForwardArgs(*a) for a in step.args]
+
+    def run(n):
+        rc = loop.moe_a2a_bench_steps(n, ctypes.byref(sets[0]), ctypes.byref(sets[1]))
+        if rc:
+            raise RuntimeError(f"moe_a2a_forward failed with code {rc}")
+
+    return run
 
 
 def summarise(per):
@@ -110,41 +144,57 @@ def main():
                       fuse_route=not args.no_fuse_route, fuse_stub=args.fuse_stub)
     x, idx, w, rs = concat_world(wl.world, dev)
 
-    def step():
-        return ata.forward(x, idx, w, rs)
-
-    y = step()
-    torch.cuda.synchronize()
-    run = step
-    use_graph = not args.no_graph
-    if use_graph:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(3):
-                step()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            y = step()
-        run = graph.replay
-
-    for _ in range(args.warmup):
-        run()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(args.steps):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    ms_per_step = e0.elapsed_time(e1) / args.steps
-
-    # per-kernel durations: eager launches, each carrying its own pair of HIP events
-    for _ in range(3):
+    # Everything runs on one non-blocking stream of its own: launches on the legacy default
+    # stream carry implicit waits on every other stream of the process.
+    main = torch.cuda.Stream()
+    main.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(main):
+        step = ata.plan(x, idx, w, rs, stream=main)  # pre-marshalled: one foreign call per step
         step()
-    per = kernel_times(lib, step, args.steps, torch)
+        y = step()  # both buffer sets exist now
+        main.synchronize()
+        run, steps_per_run = step, 1
+        use_graph = not args.no_graph
+        if use_graph:
+            # the host class alternates between two buffer sets, so one graph holds two steps
+            steps_per_run = 2
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=main):
+                step()
+                y = step()
+            run = graph.replay
+
+        n_runs = max(1, args.steps // steps_per_run)
+        timed_steps = n_runs * steps_per_run
+        # spin-up: the first milliseconds of GPU work after an idle period run below the
+        # sustained clocks; 0.3 s of untimed steps come before the W warm-up steps
+        t_spin = time.perf_counter()
+        while time.perf_counter() - t_spin < 0.3:
+            for _ in range(50):
+                run()
+            main.synchronize()
+        for _ in range(max(1, args.warmup // steps_per_run)):
+            run()
+        main.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(main)
+        for _ in range(n_runs):
+            run()
+        e1.record(main)
+        main.synchronize()
+        ms_per_step = e0.elapsed_time(e1) / timed_steps
+
+        # per-kernel durations: the same launches issued back to back from a C loop, each
+        # carrying its own pair of HIP events
+        run_n = c_loop(step)
+        run_n(4)
+        main.synchronize()
+        per = kernel_times(lib, run_n, args.steps, torch)
+        e0.record(main)
+        run_n(timed_steps)
+        e1.record(main)
+        main.synchronize()
+        eager_ms_per_step = e0.elapsed_time(e1) / timed_steps
     t_route = per_step(per, ROUTE_KERNELS, args.steps)
     t_disp = per_step(per, DISPATCH_KERNELS, args.steps)
     t_comb = per_step(per, COMBINE_KERNELS, args.steps)
@@ -165,12 +215,12 @@ def main():
                     bytes_per_launch=dom_bytes, avg_us=round(dom_us, 3), traffic=None)
 
     out = dict(
-        metric=METRIC, value=round(value, 1), unit="GB/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
+        metric=METRIC, value=round(value, 1), unit="GB/s", n_gpus=1, steps=timed_steps, warmup=args.warmup,
         ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
         dtype="fp8-e4m3 dispatch, bf16 combine" if fp8 else str(cfg.in_dtype).replace("torch.", ""),
         data="synthetic",
         config=dict(workload=args.workload, tokens=T, experts=E, top_k=K, hidden=H, emulated_ranks=W,
-                    routed_rows=T * K, combine=args.combine, launch="hipGraph replay" if use_graph else "eager",
+                    routed_rows=T * K, combine=args.combine, launch="hipGraph replay, two steps per graph" if use_graph else "eager",
                     fused_route=bool(not args.no_fuse_route and not fp8 and lib.moe_a2a_fused_ok(T, K, H)),
                     fused_stub=bool(args.fuse_stub)),
         dispatch_combine_us=round(t_dc, 3), route_us=round(t_route, 3), dispatch_us=round(t_disp, 3),
@@ -178,6 +228,7 @@ def main():
         pct_of_hbm_peak=round(100.0 * value / HBM_PEAK_GBPS, 2),
         tokens_per_s=round(T / (t_dc * 1e-6), 1),
         tokens_per_s_wall=round(T / (ms_per_step * 1e-3), 1),
+        eager_ms_per_step=round(eager_ms_per_step, 6),
         bytes=dict(dispatch=ab["dispatch"], combine=ab["combine"], stub=ab["stub"]),
         kernels=summarise(per),
         roofline=roofline,
@@ -188,17 +239,24 @@ def main():
         flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         n_cold = min(args.steps, 30)
 
-        def cold_step():
+        with torch.cuda.stream(main):
             flush.fill_(1)
-            step()
-
-        cold_step()
-        perc = kernel_times(lib, cold_step, n_cold, torch)
+            run_n(2)
+            perc = kernel_times(lib, run_n, n_cold, torch, before_each=lambda: flush.fill_(1))
         tc = per_step(perc, ROUTE_KERNELS + DISPATCH_KERNELS + COMBINE_KERNELS, n_cold)
         out["cold"] = dict(dispatch_combine_us=round(tc, 3), GBps=round(b_dc / tc / 1e3, 1),
                            pct_of_hbm_peak=round(100.0 * b_dc / tc / 1e3 / HBM_PEAK_GBPS, 2),
                            kernels={k: v["mean_us"] for k, v in summarise(perc).items()})
         del flush
+
+    if args.calibrate_copy:
+        with torch.cuda.stream(main):
+            src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(wl, mode, fp8, y, b_dc, args.cpu_seconds)

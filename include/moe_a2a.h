@@ -149,6 +149,23 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
                          int stub_kind, int E, int W, void* out, int T, int K, int H, moe_a2a_stream_t stream);
 
 /*
+ * The whole path in one call: routing + dispatch, expert stub, combine -- what custom_kernel
+ * does between reading its inputs and returning y (submission.py:192-219 of the reference;
+ * ref_kernel, all2all/reference.py:256-272).  Same kernels and results as the separate calls;
+ * one host call keeps the launches back to back.
+ *   fp8_dispatch  0 / 1          fuse_stub  0: stub kernel + combine, 1: moe_a2a_stub_combine
+ *   fuse_route    0: moe_a2a_route + dispatch, 1: moe_a2a_route_dispatch when moe_a2a_fused_ok,
+ *                 2: moe_a2a_route_dispatch whenever R fits
+ *   expert_y      [R,H] of out_type, unused (may be NULL) when fuse_stub
+ */
+int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
+                    int src_rank, int T, int K, int E, int W, int H, int in_type, int out_type, int fp8_dispatch,
+                    int stub_kind, int combine_mode, int fuse_route, int fuse_stub, int32_t* counts,
+                    int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
+                    void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
+                    size_t workspace_bytes, moe_a2a_stream_t stream);
+
+/*
  * Launch timer (opt-in, process-wide, single caller thread).  Between begin and end every
  * kernel the library launches carries a pair of HIP events bound to that dispatch, so the
  * reported time is the kernel's own begin-to-end duration on the GPU.

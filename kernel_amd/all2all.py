@@ -114,10 +114,21 @@ class HipAllToAll:
         self._bufs = {}
 
     # ---- buffers ---------------------------------------------------------------------
-    def _buffers(self, T: int, device) -> dict:
-        """Device buffers for T tokens, kept between calls (a call overwrites all of them)."""
+    def _buffers(self, T: int, device, advance: bool = False) -> dict:
+        """Device buffers for T tokens, kept between calls.
+
+        Two sets alternate (``advance=True`` at the start of a dispatch flips to the other
+        one).  Rows a kernel has just read are slow to overwrite from the next kernel, so a
+        step never writes what the step before it read; it also means the result of a call
+        stays valid until the second-next call.
+        """
         key = (T, str(device))
-        b = self._bufs.get(key)
+        ring = self._bufs.get(key)
+        if ring is None:
+            ring = self._bufs[key] = dict(sets=[None, None], cur=0)
+        if advance:
+            ring["cur"] ^= 1
+        b = ring["sets"][ring["cur"]]
         if b is not None:
             return b
         cfg = self.cfg
@@ -142,7 +153,7 @@ class HipAllToAll:
         else:
             b["disp_x"] = torch.empty(R, H, dtype=cfg.in_dtype, device=device)
             b["disp_scale"] = None
-        self._bufs[key] = b
+        ring["sets"][ring["cur"]] = b
         return b
 
     def release_buffers(self) -> None:
@@ -169,7 +180,7 @@ class HipAllToAll:
             _require_gpu(rank_start, "rank_start")
             if rank_start.dtype != torch.int32 or rank_start.numel() != W + 1:
                 raise ValueError("rank_start must be int32[world_size + 1]")
-        b = self._buffers(T, dp_x.device)
+        b = self._buffers(T, dp_x.device, advance=True)
         lib, st = self.lib, _stream()
         route_out = (_ptr(b["counts"]), _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]),
                      _ptr(b["meta"]), _ptr(b["status"]))
@@ -245,15 +256,84 @@ class HipAllToAll:
         return out_tokens
 
     # ---- whole path ------------------------------------------------------------------
+    def _forward_args(self, b: dict, x, indices, weights, rank_start, stream: int) -> tuple:
+        cfg = self.cfg
+        T, H = x.shape
+        fuse_route = 2 if self.fuse_route == "always" else int(bool(self.fuse_route))
+        return (_ptr(x), _ptr(indices), _ptr(weights), _ptr(rank_start), self.rank, T, cfg.experts_per_token,
+                cfg.num_experts, self.world_size, H, _elem(cfg.in_dtype), _elem(cfg.out_dtype), int(self.fp8_dispatch),
+                self.stub_kind, self.combine_mode, fuse_route, int(self.fuse_stub), _ptr(b["counts"]),
+                _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]), _ptr(b["meta"]),
+                _ptr(b["status"]), _ptr(b["disp_x"]), _ptr(b["disp_scale"]), _ptr(b["expert_y"]), _ptr(b["out"]),
+                _ptr(b["workspace"]), b["workspace"].numel(), stream)
+
+    def _check_inputs(self, x, indices, weights, rank_start) -> None:
+        cfg = self.cfg
+        for name, t in (("x", x), ("indices", indices), ("weights", weights)):
+            _require_gpu(t, name)
+        T, H = x.shape
+        K = cfg.experts_per_token
+        if (H != cfg.hidden_dim or tuple(indices.shape) != (T, K) or tuple(weights.shape) != (T, K)
+                or x.dtype != cfg.in_dtype or indices.dtype != torch.int32 or weights.dtype != torch.float32):
+            raise ValueError("x / indices / weights do not match the MoEConfig")
+        if rank_start is not None:
+            _require_gpu(rank_start, "rank_start")
+            if rank_start.dtype != torch.int32 or rank_start.numel() != self.world_size + 1:
+                raise ValueError("rank_start must be int32[world_size + 1]")
+
+    def _record(self, b: dict, T: int) -> Dispatched:
+        return Dispatched(self.cfg, self.world_size, T, b["counts"], b["offsets"], b["slot_of_entry"],
+                          b["src_of_slot"], b["meta"], b["disp_x"], b["disp_scale"], b["status"])
+
     def forward(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
                 rank_start: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """dispatch -> stub -> combine; returns ``y[T,H]`` (a buffer the next call reuses)."""
+        """dispatch -> stub -> combine in one library call; returns ``y[T,H]`` (a buffer the
+        second-next call reuses).  ``self.last`` holds the ``Dispatched`` record of the call."""
+        cfg = self.cfg
         if x.shape[0] == 0:
-            return torch.empty(0, self.cfg.hidden_dim, dtype=self.cfg.out_dtype, device=x.device)
-        d = self.dispatch(x, indices, rank_start)
-        if self.fuse_stub:
-            return self.stub_combine(None, weights, indices, d)
-        return self.combine(None, weights, d, self.expert_stub(d))
+            return torch.empty(0, cfg.hidden_dim, dtype=cfg.out_dtype, device=x.device)
+        self._check_inputs(x, indices, weights, rank_start)
+        b = self._buffers(x.shape[0], x.device, advance=True)
+        _lib.check(self.lib.moe_a2a_forward(*self._forward_args(b, x, indices, weights, rank_start, _stream())),
+                   "moe_a2a_forward")
+        self.last = self._record(b, x.shape[0])
+        return b["out"]
+
+    def plan(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
+             rank_start: Optional[torch.Tensor] = None, stream: Optional[torch.cuda.Stream] = None):
+        """Pre-marshalled ``forward`` for a serving loop that reuses its input tensors.
+
+        Checks shapes once and returns ``step()``: every call launches the whole path on
+        ``stream`` (default: the stream that is current NOW -- under hipGraph capture pass the
+        capturing stream), reading whatever the input tensors hold at that moment, and returns
+        ``y[T,H]``; calls alternate between the two buffer sets.  The per-call host cost is one
+        foreign call.
+        """
+        if x.shape[0] == 0:
+            raise ValueError("plan() needs at least one token")
+        self._check_inputs(x, indices, weights, rank_start)
+        T, dev = x.shape[0], x.device
+        st = stream.cuda_stream if stream is not None else _stream()
+        sets = [self._buffers(T, dev, advance=True), self._buffers(T, dev, advance=True)]
+        args = [self._forward_args(b, x, indices, weights, rank_start, st) for b in sets]
+        outs = [b["out"] for b in sets]
+        records = [self._record(b, T) for b in sets]
+        fn = self.lib.moe_a2a_forward
+        keep = (x, indices, weights, rank_start)  # the raw pointers above must stay valid
+        state = [0]
+
+        def step() -> torch.Tensor:
+            i = state[0]
+            state[0] = i ^ 1
+            rc = fn(*args[i])
+            if rc:
+                raise _lib.MoeA2AError(rc, "moe_a2a_forward")
+            self.last = records[i]
+            return outs[i]
+
+        step.inputs = keep
+        step.args = args  # the two argument tuples of moe_a2a_forward, for callers with their own loop
+        return step
 
 
 def concat_world(world: Sequence, device=None):

@@ -33,13 +33,23 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (looked on PATH and in /opt/rocm/bin)")
 
 
-def build_library(verbose: bool = False) -> str:
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *SOURCES, "-o", LIB_PATH]
+BENCH_LIB_PATH = os.path.join(PKG_DIR, "libmoe_a2a_bench.so")
+BENCH_SOURCES = [os.path.join(PKG_DIR, "csrc", "bench_loop.cpp")]
+
+
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + proc.stdout + proc.stderr)
+        raise RuntimeError("build failed:\n" + proc.stdout + proc.stderr)
+
+
+def build_library(verbose: bool = False) -> str:
+    """The product library, then the small host-loop helper bench.py uses (links against it)."""
+    _run([hipcc_path(), *HIPCC_FLAGS, *SOURCES, "-o", LIB_PATH], verbose)
+    _run(["g++", "-O2", "-shared", "-fPIC", "-I" + os.path.join(ROOT, "include"), *BENCH_SOURCES, "-o",
+          BENCH_LIB_PATH, "-L" + PKG_DIR, "-lmoe_a2a", "-Wl,-rpath,$ORIGIN"], verbose)
     return LIB_PATH
 
 

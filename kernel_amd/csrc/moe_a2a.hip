@@ -116,13 +116,17 @@ struct RouteArgs {
   int32_t* status;
 };
 
-__device__ __forceinline__ int load_expert(const RouteArgs& a, int i, bool valid) {
-  int e = valid ? a.indices[i] : 0;
+// expert id forced into [0, E); an id outside raises the caller's status flag
+__device__ __forceinline__ int clamp_expert(const RouteArgs& a, int e) {
   if (e < 0 || e >= a.E) {
     if (a.status) *a.status = 1;  // vector store; the value is the same from every lane
     e = e < 0 ? 0 : a.E - 1;
   }
   return e;
+}
+
+__device__ __forceinline__ int load_expert(const RouteArgs& a, int i, bool valid) {
+  return clamp_expert(a, valid ? a.indices[i] : 0);
 }
 
 // Lanes holding the same expert id find each other with one ballot per id bit.
@@ -379,9 +383,19 @@ __global__ __launch_bounds__(kRouteThreads) void route_rank_kernel(RouteArgs a, 
 // Scattered row stores of the dispatch always write through.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
+#ifndef MOE_A2A_THROUGH_POLICY
+#define MOE_A2A_THROUGH_POLICY 2  // tuning aid: 0 plain store, 1 non-temporal, 2 write-through
+#endif
 __device__ __forceinline__ void store_through(uint4* p, const uint4& v) {
+#if MOE_A2A_THROUGH_POLICY == 2
   u32x4_t t = {v.x, v.y, v.z, v.w};
   asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(t) : "memory");
+#elif MOE_A2A_THROUGH_POLICY == 1
+  u32x4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x4_t*>(p));
+#else
+  *p = v;
+#endif
 }
 
 template <int STREAM>
@@ -446,6 +460,7 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
   __shared__ int s_slot[MOE_A2A_MAX_TOPK];
   __shared__ int s_hist[MOE_A2A_MAX_EXPERTS];
   __shared__ int s_tmp[kFusedMaxThreads / kWave + 1];
+  __shared__ int s_starts[MOE_A2A_MAX_WORLD + 1];
   const int tid = threadIdx.x;
   const int nthreads = blockDim.x;
   const int lane = tid & (kWave - 1);
@@ -471,52 +486,53 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
     return;
   }
 
-  // every load this workgroup needs is issued here, before anything waits
   const int t = (blockIdx.x - 1) / nsplit;
   const int cs = (blockIdx.x - 1) - t * nsplit;
   const int c = cs * per + tid;
   const bool active = tid < per && c < nvec;
-  uint4 v = make_uint4(0, 0, 0, 0);
-  if (active) v = x[(size_t)t * nvec + c];
-  int ownkey = 0x7fffffff;  // lane k of every wave: key of the token's k-th entry
-  if (lane < a.K) {
-    int ik = t * a.K + lane;
-    ownkey = (load_expert(a, ik, true) << kFusedIdBits) | ik;
-  }
-  if (tid < a.K) s_slot[tid] = 0;
-
   const int chunk = nthreads * kFusedEntriesPerThread;
-  const bool vec_ok = (reinterpret_cast<uintptr_t>(a.indices) & 15u) == 0;
-  bool zeroed = false;
-  for (int i0 = 0; i0 < a.R; i0 += chunk) {
-    int key[kFusedEntriesPerThread];
+
+  // Raw expert ids of this lane's entries of the chunk starting at i0.  Indices are clamped
+  // into the table instead of branching, like every load below: with unconditional loads the
+  // compiler can wait for the early ones while the later ones stay in flight.
+  int raw[kFusedEntriesPerThread];
+  auto load_chunk = [&](int i0) {
     const int ibase = i0 + tid * kFusedEntriesPerThread;
-    if (vec_ok && ibase + kFusedEntriesPerThread <= a.R) {
-      const int4 q0 = *reinterpret_cast<const int4*>(a.indices + ibase);
-      const int e[kFusedEntriesPerThread] = {q0.x, q0.y, q0.z, q0.w};
 #pragma unroll
-      for (int m = 0; m < kFusedEntriesPerThread; ++m) {
-        int em = e[m];
-        if (em < 0 || em >= a.E) {
-          if (a.status) *a.status = 1;
-          em = em < 0 ? 0 : a.E - 1;
-        }
-        key[m] = (em << kFusedIdBits) | (ibase + m);
-      }
-    } else {
+    for (int m = 0; m < kFusedEntriesPerThread; ++m) raw[m] = a.indices[min(ibase + m, a.R - 1)];
+  };
+
+  // Counters are cleared and the barrier taken while nothing is in flight.  Then every load
+  // goes out before the first use of a loaded value: the first chunk of the table, the token's
+  // own expert ids (lane k of every wave holds entry k), the rank boundaries, and last the row
+  // itself, so that waiting for the indices (memory operations complete in order) leaves the
+  // row in flight while the slots are worked out.
+  if (tid < a.K) s_slot[tid] = 0;
+  __syncthreads();
+  load_chunk(0);
+  const int own = a.indices[t * a.K + min(lane, a.K - 1)];
+  const bool want_starts = cs == 0 && a.rank_start != nullptr;
+  const int32_t* sp = a.rank_start ? a.rank_start : a.indices;  // any readable address when unused
+  const int st0 = sp[a.rank_start ? min(tid, a.W) : 0];
+  const int st1 = sp[a.rank_start ? min(tid + nthreads, a.W) : 0];
+  __builtin_amdgcn_sched_barrier(0);  // keep the row load behind the index loads
+  const uint4 v = x[(size_t)t * nvec + min(c, nvec - 1)];
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ids outside [0, E) are clamped without branching; one flag store at the end reports them
+  bool bad = false;
+  auto key_of = [&](int e, int i) {
+    bad |= e < 0 || e >= a.E;
+    return (min(max(e, 0), a.E - 1) << kFusedIdBits) | i;
+  };
+  const int ownkey = lane < a.K ? key_of(own, t * a.K + lane) : 0x7fffffff;
+  // one chunk: count, for each of the token's K keys, the smaller keys this wave holds
+  auto count_chunk = [&](int i0) {
+    const int ibase = i0 + tid * kFusedEntriesPerThread;
+    int key[kFusedEntriesPerThread];
 #pragma unroll
-      for (int m = 0; m < kFusedEntriesPerThread; ++m) {
-        int i = ibase + m;
-        bool valid = i < a.R;
-        int e = load_expert(a, i, valid);
-        key[m] = valid ? ((e << kFusedIdBits) | i) : 0x7fffffff;
-      }
-    }
-    if (!zeroed) {
-      __syncthreads();  // counters are zero before the first add
-      zeroed = true;
-    }
-    if (__ballot(ibase < a.R) == 0) continue;  // this wave holds no entries of the chunk
+    for (int m = 0; m < kFusedEntriesPerThread; ++m) key[m] = ibase + m < a.R ? key_of(raw[m], ibase + m) : 0x7fffffff;
+    if (__ballot(ibase < a.R) == 0) return;  // this wave holds no entries of the chunk
     for (int k = 0; k < a.K; ++k) {
       const int mykey = __builtin_amdgcn_readlane(ownkey, k);
       int cnt = 0;
@@ -524,6 +540,16 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
       for (int m = 0; m < kFusedEntriesPerThread; ++m) cnt += __popcll(__ballot(key[m] < mykey));
       if (lane == 0 && cnt) atomicAdd(&s_slot[k], cnt);
     }
+  };
+  count_chunk(0);  // outside the loop: only here are the row and rank loads still in flight
+  for (int i0 = chunk; i0 < a.R; i0 += chunk) {
+    load_chunk(i0);
+    count_chunk(i0);
+  }
+  if (bad && a.status) *a.status = 1;
+  if (want_starts) {  // W + 1 <= 257 <= 2 * nthreads
+    if (tid <= a.W) s_starts[tid] = st0;
+    if (tid + nthreads <= a.W) s_starts[tid + nthreads] = st1;
   }
   __syncthreads();
 
@@ -534,16 +560,8 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
     const int slot = s_slot[tid];
     a.slot_of_entry[i] = slot;
     a.src_of_slot[slot] = i;
-    int sr = a.src_rank, tl = t;
-    if (a.rank_start) {
-      int lo = 0, hi = a.W;
-      while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (a.rank_start[mid] <= t) lo = mid; else hi = mid;
-      }
-      sr = lo;
-      tl = t - a.rank_start[lo];
-    }
+    int sr, tl;
+    locate_token(s_starts, a.W, a.src_rank, a.rank_start != nullptr, t, sr, tl);
     int32_t* m = a.meta + (size_t)slot * MOE_A2A_META_DIM;
     m[0] = ownkey >> kFusedIdBits;
     m[1] = sr;
@@ -1264,6 +1282,39 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
 #undef SC_LAUNCH
 }
 #undef MOE_A2A_SWITCH_KT
+
+int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
+                    int src_rank, int T, int K, int E, int W, int H, int in_type, int out_type, int fp8_dispatch,
+                    int stub_kind, int combine_mode, int fuse_route, int fuse_stub, int32_t* counts,
+                    int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
+                    void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
+                    size_t workspace_bytes, moe_a2a_stream_t stream) {
+  if (!known_type(in_type) || !known_type(out_type)) return MOE_A2A_E_DTYPE;
+  if (fp8_dispatch && !disp_scale) return MOE_A2A_E_NULL;
+  if (!fuse_stub && T > 0 && !expert_y) return MOE_A2A_E_NULL;
+  const bool fused = !fp8_dispatch && (fuse_route == 2 ? (T > 0 && (long long)T * K <= kFusedMaxRows)
+                                                         : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
+  if (fused) {
+    if (int rc = moe_a2a_route_dispatch(x, indices, rank_start, src_rank, T, K, E, W, H, counts, offsets,
+                                        slot_of_entry, src_of_slot, meta, status, disp, stream))
+      return rc;
+  } else {
+    if (int rc = moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, counts, offsets, slot_of_entry,
+                               src_of_slot, meta, status, workspace, workspace_bytes, stream))
+      return rc;
+    if (int rc = fp8_dispatch ? moe_a2a_dispatch_fp8(x, in_type, slot_of_entry, (uint8_t*)disp, disp_scale, T, K, H,
+                                                     stream)
+                              : moe_a2a_dispatch(x, slot_of_entry, disp, T, K, H, stream))
+      return rc;
+  }
+  const float* scale = fp8_dispatch ? disp_scale : nullptr;
+  if (fuse_stub)
+    return moe_a2a_stub_combine(disp, scale, indices, weights, slot_of_entry, combine_mode, in_type, out_type,
+                                stub_kind, E, W, out, T, K, H, stream);
+  if (int rc = moe_a2a_stub(disp, scale, meta, in_type, out_type, stub_kind, E, W, expert_y, T * K, H, stream))
+    return rc;
+  return moe_a2a_combine(expert_y, weights, slot_of_entry, combine_mode, out_type, out, T, K, H, stream);
+}
 
 int moe_a2a_timer_begin(int capacity) {
   if (g_timer.active || capacity < 1) return MOE_A2A_E_STATE;

@@ -35,5 +35,5 @@ def custom_kernel(data, stub_kind: int = STUB_OWNER_RANK, combine_mode: int = CO
     ata = _instance(cfg, rank, world_size, x.device, stub_kind, combine_mode)
     with torch.cuda.device(x.device):
         y = ata.forward(x.contiguous(), rank_data.indices.contiguous(), rank_data.weights.contiguous())
-    # the caller owns its result (eval.py deletes it after each run): hand out a copy of the reused buffer
+    # the caller owns its result (eval.py deletes it after each run): hand out a copy of the ring buffer
     return y[: rank_data.num_tokens].clone()

@@ -154,6 +154,26 @@ def test_limits_and_generic_topk(gpu_device, E, K, T, H):
             compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, combine_mode=mode, fuse_route=fuse)
 
 
+@pytest.mark.parametrize("name", ["tiny", "dsv3_rank", "skew_world"])
+def test_forward_single_call_equals_separate_calls(gpu_device, name):
+    wl = C.generate_workload(name)
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    want = V.run_world(wl.cfg, wl.world, stub_kind=wl.stub_kind)
+    for fuse_route in ("always", True, False):
+        for fuse_stub in (False, True):
+            ata = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fuse_route=fuse_route,
+                              fuse_stub=fuse_stub)
+            for _ in range(3):  # both buffer sets, and the first one again
+                y = ata.forward(x, idx, w, rs)
+                assert_same("y", y, want["y"])
+                assert_same("meta", ata.last.meta, want["meta"])
+                assert_same("disp_x", ata.last.disp_x, want["disp_x"])
+            step = ata.plan(x, idx, w, rs)
+            for _ in range(3):
+                assert_same("y (planned)", step(), want["y"])
+                assert_same("slot_of_entry (planned)", ata.last.slot_of_entry, want["slot_of_entry"])
+
+
 def test_custom_kernel_contract(gpu_device):
     """custom_kernel(data) per rank == oracle ref_kernel, checked with the reference's tolerance."""
     from kernel_amd.submission import custom_kernel
