@@ -90,7 +90,7 @@ def kernel_times(lib, run_n, steps, torch, before_each=None):
 class ForwardArgs(ctypes.Structure):
     """Mirror of moe_a2a_forward_args in kernel_amd/csrc/bench_loop.cpp."""
     _fields_ = ([(n, ctypes.c_void_p) for n in ("x", "indices", "weights", "rank_start")] +
-                [(n, ctypes.c_int) for n in ("src_rank", "T", "K", "E", "W", "H", "in_type", "out_type", "fp8_dispatch",
+                [(n, ctypes.c_int) for n in ("src_rank", "T", "K", "E", "W", "H", "max_recv", "in_type", "out_type", "fp8_dispatch",
                                              "stub_kind", "combine_mode", "fuse_route", "fuse_stub")] +
                 [(n, ctypes.c_void_p) for n in ("counts", "offsets", "slot_of_entry", "src_of_slot", "meta", "status",
                                                 "disp", "disp_scale", "expert_y", "out", "workspace")] +

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MOE_A2A_ABI_VERSION 1
+#define MOE_A2A_ABI_VERSION 2
 
 /* element types of activations */
 #define MOE_A2A_F16 0
@@ -85,10 +85,20 @@ size_t moe_a2a_workspace_bytes(int T, int K, int E);
  *                        (all2all/reference.py:85)
  *   status               optional int32[1]: set to 1 if an expert id was out of range
  *                        (such ids are clamped into [0,E) so no access goes out of bounds)
+ *   max_recv             0: compact layout, rows of all experts back to back (R rows).
+ *                        > 0: the reference's padded layout (all2all/reference.py:65,127-136):
+ *                        expert e owns rows [e*max_recv, (e+1)*max_recv), its j-th entry sits at
+ *                        e*max_recv + j, so disp_x / meta / src_of_slot have E*max_recv rows and,
+ *                        viewed as [W, E_l, max_recv, .], are the expert_x / expert_meta of every
+ *                        owner rank; rows past counts[e] are not written.  slot_of_entry then
+ *                        holds these physical rows, which is all dispatch and combine follow.
+ *                        An expert with more than max_recv entries sets status to 2 (the extra
+ *                        entries are folded onto the segment's last row).
  */
 int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
-                  int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
-                  int32_t* status, void* workspace, size_t workspace_bytes, moe_a2a_stream_t stream);
+                  int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
+                  int32_t* meta, int32_t* status, void* workspace, size_t workspace_bytes,
+                  moe_a2a_stream_t stream);
 
 /*
  * Dispatch: disp_x[slot_of_entry[t*K+k], :] = x[t, :] for every k.  Each token row is read
@@ -108,9 +118,9 @@ int moe_a2a_fused_max_rows(void);
  * above and a routing table small enough that re-reading it in every workgroup stays cheap. */
 int moe_a2a_fused_ok(int T, int K, int H);
 int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
-                           int K, int E, int W, int H, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
-                           int32_t* src_of_slot, int32_t* meta, int32_t* status, void* disp_x,
-                           moe_a2a_stream_t stream);
+                           int K, int E, int W, int H, int max_recv, int32_t* counts, int32_t* offsets,
+                           int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
+                           void* disp_x, moe_a2a_stream_t stream);
 
 /*
  * fp8 dispatch: quantise each token row once to e4m3fn with one f32 scale per 128 columns
@@ -125,9 +135,12 @@ int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry
 /*
  * Expert stub (all2all/reference.py:262): y[row,:] = round_out(f32(round_out(x[row,:])) * s(e)),
  * e = meta[row,0].  With disp_scale != NULL the input is fp8: y = round_out((f32(q)*scale) * s(e)).
+ * rows == NULL: rows 0..R-1 (compact layout).  rows != NULL: the R rows rows[0..R-1] -- pass
+ * slot_of_entry for the padded layout, so that only rows holding an entry are touched (the
+ * reference multiplies the whole padded buffer, uninitialised rows included).
  */
-int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta, int in_type, int out_type,
-                 int stub_kind, int E, int W, void* y, int R, int H, moe_a2a_stream_t stream);
+int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta, const int32_t* rows, int in_type,
+                 int out_type, int stub_kind, int E, int W, void* y, int R, int H, moe_a2a_stream_t stream);
 
 /*
  * Combine: out[t,:] = sum_k weights[t,k] * expert_y[slot_of_entry[t*K+k], :]
@@ -156,13 +169,14 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
  *   fp8_dispatch  0 / 1          fuse_stub  0: stub kernel + combine, 1: moe_a2a_stub_combine
  *   fuse_route    0: moe_a2a_route + dispatch, 1: moe_a2a_route_dispatch when moe_a2a_fused_ok,
  *                 2: moe_a2a_route_dispatch whenever R fits
- *   expert_y      [R,H] of out_type, unused (may be NULL) when fuse_stub
+ *   expert_y      [R,H] (padded layout: [E*max_recv,H]) of out_type, unused (may be NULL) when fuse_stub
+ *   max_recv      0 compact layout, > 0 padded layout (see moe_a2a_route)
  */
 int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
-                    int src_rank, int T, int K, int E, int W, int H, int in_type, int out_type, int fp8_dispatch,
-                    int stub_kind, int combine_mode, int fuse_route, int fuse_stub, int32_t* counts,
-                    int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
-                    void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
+                    int src_rank, int T, int K, int E, int W, int H, int max_recv, int in_type, int out_type,
+                    int fp8_dispatch, int stub_kind, int combine_mode, int fuse_route, int fuse_stub,
+                    int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
+                    int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
                     size_t workspace_bytes, moe_a2a_stream_t stream);
 
 /*

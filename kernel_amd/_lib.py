@@ -9,7 +9,7 @@ import os
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmoe_a2a.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 F16, BF16 = 0, 1
 
 _i32p = C.c_void_p  # device pointers travel as plain addresses
@@ -21,19 +21,19 @@ PROTOTYPES = {
     "moe_a2a_abi_version": (_int, []),
     "moe_a2a_strerror": (C.c_char_p, [_int]),
     "moe_a2a_workspace_bytes": (C.c_size_t, [_int, _int, _int]),
-    "moe_a2a_route": (_int, [_i32p, _i32p, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p, _i32p, _i32p, _i32p,
-                             _vp, C.c_size_t, _vp]),
+    "moe_a2a_route": (_int, [_i32p, _i32p, _int, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p, _i32p, _i32p,
+                             _i32p, _vp, C.c_size_t, _vp]),
     "moe_a2a_dispatch": (_int, [_vp, _i32p, _vp, _int, _int, _int, _vp]),
     "moe_a2a_fused_max_rows": (_int, []),
     "moe_a2a_fused_ok": (_int, [_int, _int, _int]),
-    "moe_a2a_route_dispatch": (_int, [_vp, _i32p, _i32p, _int, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p,
-                                      _i32p, _i32p, _i32p, _vp, _vp]),
+    "moe_a2a_route_dispatch": (_int, [_vp, _i32p, _i32p, _int, _int, _int, _int, _int, _int, _int, _i32p, _i32p,
+                                      _i32p, _i32p, _i32p, _i32p, _vp, _vp]),
     "moe_a2a_dispatch_fp8": (_int, [_vp, _int, _i32p, _vp, _vp, _int, _int, _int, _vp]),
-    "moe_a2a_stub": (_int, [_vp, _vp, _i32p, _int, _int, _int, _int, _int, _vp, _int, _int, _vp]),
+    "moe_a2a_stub": (_int, [_vp, _vp, _i32p, _i32p, _int, _int, _int, _int, _int, _vp, _int, _int, _vp]),
     "moe_a2a_combine": (_int, [_vp, _vp, _i32p, _int, _int, _vp, _int, _int, _int, _vp]),
     "moe_a2a_stub_combine": (_int, [_vp, _vp, _i32p, _vp, _i32p, _int, _int, _int, _int, _int, _int, _vp, _int, _int,
                                     _int, _vp]),
-    "moe_a2a_forward": (_int, [_vp, _i32p, _vp, _i32p] + [_int] * 13 + [_i32p] * 6 + [_vp, _vp, _vp, _vp, _vp, C.c_size_t,
+    "moe_a2a_forward": (_int, [_vp, _i32p, _vp, _i32p] + [_int] * 14 + [_i32p] * 6 + [_vp, _vp, _vp, _vp, _vp, C.c_size_t,
                                                                                       _vp]),
     "moe_a2a_timer_begin": (_int, [_int]),
     "moe_a2a_timer_end": (_int, [C.POINTER(C.c_int), C.POINTER(C.c_float), _int]),

@@ -5,9 +5,11 @@
 ``combine``.  Differences from the reference that a caller sees:
 
 * one GPU holds every destination rank, so ``dispatch`` returns the rows of ALL
-  ``num_experts`` experts in one compact expert-major buffer (``Dispatched``) instead of
-  the calling rank's padded ``[E_l, max_recv, H]`` slice; ``Dispatched.padded(owner)``
-  rebuilds the reference's triple for one owner rank;
+  ``num_experts`` experts in one expert-major buffer (``Dispatched``): compact by default
+  (rows back to back), or with ``padded=True`` exactly the reference's ``[E_l, max_recv, .]``
+  buffers of every owner rank laid end to end; ``Dispatched.padded(owner)`` hands out the
+  reference's ``(expert_num_tokens, expert_x, expert_meta)`` triple of one owner rank
+  (views in the padded layout, a copy in the compact one);
 * there is no process group: the three exchanges per phase are gone;
 * ``combine`` writes ``out[:T]`` (it does not add into what ``out`` held before).
 
@@ -63,7 +65,8 @@ class Dispatched:
     meta: torch.Tensor  # [R,5] int32: e, source rank, token in rank, k, 0
     disp_x: torch.Tensor  # [R,H] in_dtype, or uint8 e4m3fn bits for fp8 dispatch
     disp_scale: Optional[torch.Tensor] = None  # [R,H/128] f32 (fp8 only)
-    status: Optional[torch.Tensor] = None  # [1] int32, 1 if an expert id was out of range
+    status: Optional[torch.Tensor] = None  # [1] int32: 1 expert id out of range, 2 padded segment overflow
+    max_recv: int = 0  # > 0: padded layout, expert e owns rows [e*max_recv, (e+1)*max_recv)
 
     @property
     def num_rows(self) -> int:
@@ -74,8 +77,16 @@ class Dispatched:
         padded shape (all2all/reference.py:123-148); rows past the count are zero."""
         cfg, W = self.cfg, self.world_size
         E_l = cfg.num_experts // W
-        max_recv = max_recv if max_recv is not None else cfg.max_num_tokens * W
         lo, hi = owner_rank * E_l, (owner_rank + 1) * E_l
+        if self.max_recv > 0 and max_recv in (None, self.max_recv):
+            # already laid out that way: views, no copy (rows past the counts are uninitialised,
+            # as they are in the reference)
+            H = self.disp_x.shape[1]
+            return (self.counts[lo:hi], self.disp_x.view(W, E_l, self.max_recv, H)[owner_rank],
+                    self.meta.view(W, E_l, self.max_recv, META_DIM)[owner_rank])
+        if self.max_recv > 0:
+            raise ValueError("this record is padded with a different max_recv")
+        max_recv = max_recv if max_recv is not None else cfg.max_num_tokens * W
         num = self.counts[lo:hi].clone()
         off = self.offsets[lo:hi + 1].tolist()
         ex = torch.zeros(E_l, max_recv, self.disp_x.shape[1], dtype=self.disp_x.dtype, device=self.disp_x.device)
@@ -96,14 +107,15 @@ class HipAllToAll:
 
     def __init__(self, cfg: MoEConfig, rank: int, world_size: int, stub_kind: int = STUB_OWNER_RANK,
                  combine_mode: int = COMBINE_STRICT, fp8_dispatch: bool = False, fuse_route: bool = True,
-                 fuse_stub: bool = False):
+                 fuse_stub: bool = False, padded: bool = False, max_recv: Optional[int] = None):
         if cfg.num_experts % world_size:
             raise ValueError("num_experts must be a multiple of world_size")
         self.cfg = cfg
         self.rank = rank
         self.world_size = world_size
         self.num_local_experts = cfg.num_experts // world_size
-        self.max_recv = cfg.max_num_tokens * world_size
+        self.max_recv = max_recv if max_recv is not None else cfg.max_num_tokens * world_size
+        self.padded = padded  # rows laid out as the reference's [E_l, max_recv, .] buffers of every owner rank
         self.stub_kind = stub_kind
         self.combine_mode = combine_mode
         self.fp8_dispatch = fp8_dispatch
@@ -134,24 +146,25 @@ class HipAllToAll:
         cfg = self.cfg
         K, H, E = cfg.experts_per_token, cfg.hidden_dim, cfg.num_experts
         R = T * K
+        rows = E * self.max_recv if self.padded else R  # rows of the dispatched buffers
         i32 = dict(dtype=torch.int32, device=device)
         b = dict(
             counts=torch.empty(E, **i32),
             offsets=torch.empty(E + 1, **i32),
             slot_of_entry=torch.empty(R, **i32),
-            src_of_slot=torch.empty(R, **i32),
-            meta=torch.empty(R, META_DIM, **i32),
+            src_of_slot=torch.empty(rows, **i32),
+            meta=torch.empty(rows, META_DIM, **i32),
             status=torch.zeros(1, **i32),
             workspace=torch.empty(max(self.lib.moe_a2a_workspace_bytes(T, K, E), 256), dtype=torch.uint8,
                                   device=device),
-            expert_y=torch.empty(R, H, dtype=cfg.out_dtype, device=device),
+            expert_y=torch.empty(rows, H, dtype=cfg.out_dtype, device=device),
             out=torch.empty(T, H, dtype=cfg.out_dtype, device=device),
         )
         if self.fp8_dispatch:
-            b["disp_x"] = torch.empty(R, H, dtype=torch.uint8, device=device)
-            b["disp_scale"] = torch.empty(R, H // FP8_BLOCK, dtype=torch.float32, device=device)
+            b["disp_x"] = torch.empty(rows, H, dtype=torch.uint8, device=device)
+            b["disp_scale"] = torch.empty(rows, H // FP8_BLOCK, dtype=torch.float32, device=device)
         else:
-            b["disp_x"] = torch.empty(R, H, dtype=cfg.in_dtype, device=device)
+            b["disp_x"] = torch.empty(rows, H, dtype=cfg.in_dtype, device=device)
             b["disp_scale"] = None
         ring["sets"][ring["cur"]] = b
         return b
@@ -182,15 +195,16 @@ class HipAllToAll:
                 raise ValueError("rank_start must be int32[world_size + 1]")
         b = self._buffers(T, dp_x.device, advance=True)
         lib, st = self.lib, _stream()
+        pad = self.max_recv if self.padded else 0
         route_out = (_ptr(b["counts"]), _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]),
                      _ptr(b["meta"]), _ptr(b["status"]))
         if self.fuse_route and not self.fp8_dispatch and (
                 self.fuse_route == "always" and 0 < T * K <= self._fused_max_rows
                 or self.lib.moe_a2a_fused_ok(T, K, H)):
             _lib.check(lib.moe_a2a_route_dispatch(_ptr(dp_x), _ptr(indices), _ptr(rank_start), self.rank, T, K, E, W,
-                                                  H, *route_out, _ptr(b["disp_x"]), st), "moe_a2a_route_dispatch")
+                                                  H, pad, *route_out, _ptr(b["disp_x"]), st), "moe_a2a_route_dispatch")
         else:
-            _lib.check(lib.moe_a2a_route(_ptr(indices), _ptr(rank_start), self.rank, T, K, E, W, *route_out,
+            _lib.check(lib.moe_a2a_route(_ptr(indices), _ptr(rank_start), self.rank, T, K, E, W, pad, *route_out,
                                          _ptr(b["workspace"]), b["workspace"].numel(), st), "moe_a2a_route")
             if self.fp8_dispatch:
                 _lib.check(lib.moe_a2a_dispatch_fp8(_ptr(dp_x), _elem(cfg.in_dtype), _ptr(b["slot_of_entry"]),
@@ -200,16 +214,17 @@ class HipAllToAll:
                 _lib.check(lib.moe_a2a_dispatch(_ptr(dp_x), _ptr(b["slot_of_entry"]), _ptr(b["disp_x"]), T, K, H, st),
                            "moe_a2a_dispatch")
         return Dispatched(cfg, W, T, b["counts"], b["offsets"], b["slot_of_entry"], b["src_of_slot"], b["meta"],
-                          b["disp_x"], b["disp_scale"], b["status"])
+                          b["disp_x"], b["disp_scale"], b["status"], pad)
 
     # ---- expert stub -----------------------------------------------------------------
     def expert_stub(self, d: Dispatched) -> torch.Tensor:
         """all2all/reference.py:262 on the compact rows -> ``expert_y[R,H]`` out_dtype."""
         cfg = self.cfg
-        R, H = d.disp_x.shape
+        R, H = d.num_rows, d.disp_x.shape[1]
         y = self._buffers(d.num_tokens, d.disp_x.device)["expert_y"]
         in_type = _lib.BF16 if d.disp_scale is not None else _elem(d.disp_x.dtype)
-        _lib.check(self.lib.moe_a2a_stub(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(d.meta), in_type,
+        rows = d.slot_of_entry if d.max_recv > 0 else None  # padded: only rows that hold an entry
+        _lib.check(self.lib.moe_a2a_stub(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(d.meta), _ptr(rows), in_type,
                                          _elem(cfg.out_dtype), self.stub_kind, cfg.num_experts, self.world_size,
                                          _ptr(y), R, H, _stream()), "moe_a2a_stub")
         return y
@@ -225,8 +240,8 @@ class HipAllToAll:
         _require_gpu(expert_y, "expert_y")
         if weights.dtype != torch.float32 or tuple(weights.shape) != (T, K):
             raise ValueError("weights must be float32[T,K]")
-        if expert_y.dtype != cfg.out_dtype or tuple(expert_y.shape) != (T * K, H):
-            raise ValueError("expert_y must be out_dtype[T*K,H]")
+        if expert_y.dtype != cfg.out_dtype or tuple(expert_y.shape) != (d.disp_x.shape[0], H):
+            raise ValueError("expert_y must be out_dtype[rows,H] with the rows of the dispatched buffer")
         if out_tokens is None:
             out_tokens = self._buffers(T, expert_y.device)["out"]
         else:
@@ -261,7 +276,7 @@ class HipAllToAll:
         T, H = x.shape
         fuse_route = 2 if self.fuse_route == "always" else int(bool(self.fuse_route))
         return (_ptr(x), _ptr(indices), _ptr(weights), _ptr(rank_start), self.rank, T, cfg.experts_per_token,
-                cfg.num_experts, self.world_size, H, _elem(cfg.in_dtype), _elem(cfg.out_dtype), int(self.fp8_dispatch),
+                cfg.num_experts, self.world_size, H, self.max_recv if self.padded else 0, _elem(cfg.in_dtype), _elem(cfg.out_dtype), int(self.fp8_dispatch),
                 self.stub_kind, self.combine_mode, fuse_route, int(self.fuse_stub), _ptr(b["counts"]),
                 _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]), _ptr(b["meta"]),
                 _ptr(b["status"]), _ptr(b["disp_x"]), _ptr(b["disp_scale"]), _ptr(b["expert_y"]), _ptr(b["out"]),
@@ -283,7 +298,8 @@ class HipAllToAll:
 
     def _record(self, b: dict, T: int) -> Dispatched:
         return Dispatched(self.cfg, self.world_size, T, b["counts"], b["offsets"], b["slot_of_entry"],
-                          b["src_of_slot"], b["meta"], b["disp_x"], b["disp_scale"], b["status"])
+                          b["src_of_slot"], b["meta"], b["disp_x"], b["disp_scale"], b["status"],
+                          self.max_recv if self.padded else 0)
 
     def forward(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
                 rank_start: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -108,6 +108,7 @@ struct RouteArgs {
   int src_rank;
   int T, K, E, W, R;
   int nbits;  // bits needed for an expert id
+  int pad;    // 0: compact rows; > 0: rows of expert e start at e * pad (the reference's max_recv)
   int32_t* counts;
   int32_t* offsets;
   int32_t* slot_of_entry;
@@ -191,7 +192,22 @@ __device__ __forceinline__ void locate_token(const int* starts, int W, int src_r
   local = t - starts[lo];
 }
 
-__device__ __forceinline__ void emit_entry(const RouteArgs& a, const int* starts, int i, int e, int slot) {
+// Row of the entry that is the j-th of expert e, where its compact slot is first_of_e + j.
+// Padded layout: a segment holds `pad` rows; an entry beyond that is folded onto the last
+// row of its segment and reported through the status flag (2) -- no access leaves the buffer.
+__device__ __forceinline__ int row_of(const RouteArgs& a, int e, int slot, int first_of_e) {
+  if (a.pad == 0) return slot;
+  int j = slot - first_of_e;
+  if (j >= a.pad) {
+    if (a.status) *a.status = 2;
+    j = a.pad - 1;
+  }
+  return e * a.pad + j;
+}
+
+__device__ __forceinline__ void emit_entry(const RouteArgs& a, const int* starts, int i, int e, int slot_compact,
+                                           int first_of_e) {
+  const int slot = row_of(a, e, slot_compact, first_of_e);
   a.slot_of_entry[i] = slot;
   a.src_of_slot[slot] = i;
   int t = i / a.K;
@@ -271,9 +287,10 @@ __global__ __launch_bounds__(kRouteThreads) void route_tiles_kernel(RouteArgs a)
       wcnt[w * a.E + tid] = run;
       run += c;
     }
+    rest[tid] = excl;  // rest[] is not needed any more: it now holds the first slot of each expert
   }
   __syncthreads();
-  if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank);
+  if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank, rest[e]);
 }
 
 // Routing in three launches for larger tables.
@@ -363,7 +380,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_rank_kernel(RouteArgs a, 
     }
   }
   __syncthreads();
-  if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank);
+  if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank, a.pad ? a.offsets[e] : 0);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -534,10 +551,13 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
     for (int m = 0; m < kFusedEntriesPerThread; ++m) key[m] = ibase + m < a.R ? key_of(raw[m], ibase + m) : 0x7fffffff;
     if (__ballot(ibase < a.R) == 0) return;  // this wave holds no entries of the chunk
     for (int k = 0; k < a.K; ++k) {
-      const int mykey = __builtin_amdgcn_readlane(ownkey, k);
+      // compact: keys below mine; padded: keys below mine of my own expert (position in segment)
+      const unsigned mykey = (unsigned)__builtin_amdgcn_readlane(ownkey, k);
+      const unsigned lo = a.pad ? (mykey & ~((1u << kFusedIdBits) - 1u)) : 0u;
+      const unsigned span = mykey - lo;
       int cnt = 0;
 #pragma unroll
-      for (int m = 0; m < kFusedEntriesPerThread; ++m) cnt += __popcll(__ballot(key[m] < mykey));
+      for (int m = 0; m < kFusedEntriesPerThread; ++m) cnt += __popcll(__ballot((unsigned)key[m] - lo < span));
       if (lane == 0 && cnt) atomicAdd(&s_slot[k], cnt);
     }
   };
@@ -553,6 +573,10 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
   }
   __syncthreads();
 
+  if (a.pad) {  // position in segment -> row of the padded layout (counts are final here)
+    if (tid < a.K) s_slot[tid] = row_of(a, ownkey >> kFusedIdBits, s_slot[tid], 0);
+    __syncthreads();
+  }
   if (active)
     for (int k = 0; k < a.K; ++k) store_through(disp + (size_t)s_slot[k] * nvec + c, v);
   if (cs == 0 && tid < a.K) {
@@ -663,12 +687,14 @@ template <class In, class Out, int STREAM>
 __global__ __launch_bounds__(kRowMaxThreads) void stub_rows_kernel(const uint4* __restrict__ disp,
                                                                     const int32_t* __restrict__ meta,
                                                                     uint4* __restrict__ y, int stub_kind, int E,
-                                                                    int E_l, int nvec, int per, int nsplit) {
+                                                                    int E_l, int nvec, int per, int nsplit,
+                                                                    const int32_t* __restrict__ rows) {
   const RowCut r = row_cut(nvec, per, nsplit);
   if (!r.active) return;
-  const uint4 v = load_row<STREAM>(disp + (size_t)r.t * nvec + r.c);
-  const float s = stub_factor(meta[(size_t)r.t * MOE_A2A_META_DIM], stub_kind, E, E_l);
-  store_row<STREAM>(y + (size_t)r.t * nvec + r.c, stub_vec<In, Out>(v, s));
+  const size_t row = rows ? rows[r.t] : r.t;  // padded layout: visit the rows that hold entries
+  const uint4 v = load_row<STREAM>(disp + row * nvec + r.c);
+  const float s = stub_factor(meta[row * MOE_A2A_META_DIM], stub_kind, E, E_l);
+  store_row<STREAM>(y + row * nvec + r.c, stub_vec<In, Out>(v, s));
 }
 
 // fp8 rows: each lane turns 8 bytes into 8 output elements, so a wave's stores are one
@@ -679,10 +705,12 @@ __global__ __launch_bounds__(kRowMaxThreads) void stub_fp8_kernel(const uint2* _
                                                                    const float* __restrict__ disp_scale,
                                                                    const int32_t* __restrict__ meta,
                                                                    uint4* __restrict__ y, int stub_kind, int E,
-                                                                   int E_l, int nvec, int per, int nsplit) {
+                                                                   int E_l, int nvec, int per, int nsplit,
+                                                                   const int32_t* __restrict__ rows) {
   const RowCut r = row_cut(nvec, per, nsplit);
   if (!r.active) return;
-  const uint2* src = disp_q + (size_t)r.t * nvec + r.c;
+  const size_t row = rows ? rows[r.t] : r.t;
+  const uint2* src = disp_q + row * nvec + r.c;
   uint2 q;
   if (STREAM) {
     typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
@@ -691,12 +719,12 @@ __global__ __launch_bounds__(kRowMaxThreads) void stub_fp8_kernel(const uint2* _
   } else {
     q = *src;
   }
-  const float scale = disp_scale[(size_t)r.t * (nvec >> 4) + (r.c >> 4)];
-  const float s = stub_factor(meta[(size_t)r.t * MOE_A2A_META_DIM], stub_kind, E, E_l);
+  const float scale = disp_scale[row * (nvec >> 4) + (r.c >> 4)];
+  const float s = stub_factor(meta[row * MOE_A2A_META_DIM], stub_kind, E, E_l);
   float f0[4], f1[4];
   fp8x4_to_f32(q.x, f0);
   fp8x4_to_f32(q.y, f1);
-  store_row<STREAM>(y + (size_t)r.t * nvec + r.c,
+  store_row<STREAM>(y + row * nvec + r.c,
                     make_uint4(Out::pack((f0[0] * scale) * s, (f0[1] * scale) * s),
                                Out::pack((f0[2] * scale) * s, (f0[3] * scale) * s),
                                Out::pack((f1[0] * scale) * s, (f1[1] * scale) * s),
@@ -993,14 +1021,16 @@ size_t moe_a2a_workspace_bytes(int T, int K, int E) {
 }
 
 int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
-                  int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
-                  int32_t* status, void* workspace, size_t workspace_bytes, moe_a2a_stream_t stream_) {
+                  int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
+                  int32_t* meta, int32_t* status, void* workspace, size_t workspace_bytes,
+                  moe_a2a_stream_t stream_) {
   if (int rc = check_route_shape(T, K, E, W)) return rc;
+  if (max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
   if (!counts || !offsets) return MOE_A2A_E_NULL;
   if (T > 0 && (!indices || !slot_of_entry || !src_of_slot || !meta)) return MOE_A2A_E_NULL;
   hipStream_t stream = (hipStream_t)stream_;
-  RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), counts, offsets, slot_of_entry,
-              src_of_slot, meta, status};
+  RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
+              slot_of_entry, src_of_slot, meta, status};
   const size_t lds_w = (size_t)kRouteWaves * E * sizeof(int);
   const size_t lds_starts = (size_t)(W + 1) * sizeof(int);
   if (a.R <= kRouteTilesMaxRows) {
@@ -1066,16 +1096,17 @@ int moe_a2a_fused_ok(int T, int K, int H) {
 }
 
 int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
-                           int K, int E, int W, int H, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
-                           int32_t* src_of_slot, int32_t* meta, int32_t* status, void* disp_x,
-                           moe_a2a_stream_t stream_) {
+                           int K, int E, int W, int H, int max_recv, int32_t* counts, int32_t* offsets,
+                           int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
+                           void* disp_x, moe_a2a_stream_t stream_) {
   if (int rc = check_route_shape(T, K, E, W)) return rc;
+  if (max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
   if ((long long)T * K > kFusedMaxRows) return MOE_A2A_E_SHAPE;
   if (int rc = check_rows(x, disp_x, T, K, H, 8)) return rc;
   if (!counts || !offsets) return MOE_A2A_E_NULL;
   if (T > 0 && (!indices || !slot_of_entry || !src_of_slot || !meta)) return MOE_A2A_E_NULL;
-  RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), counts, offsets, slot_of_entry,
-              src_of_slot, meta, status};
+  RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
+              slot_of_entry, src_of_slot, meta, status};
   const int nvec = H / 8;
   const RowGeom g = row_geom(nvec, 1, kFusedMaxThreads, 256);
   return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel, dim3((unsigned)T * g.nsplit + 1), dim3(g.threads), 0,
@@ -1107,8 +1138,8 @@ int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry
 
 static bool known_type(int t) { return t == MOE_A2A_F16 || t == MOE_A2A_BF16; }
 
-int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta, int in_type, int out_type,
-                 int stub_kind, int E, int W, void* y, int R, int H, moe_a2a_stream_t stream_) {
+int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta, const int32_t* rows, int in_type,
+                 int out_type, int stub_kind, int E, int W, void* y, int R, int H, moe_a2a_stream_t stream_) {
   if (!known_type(out_type) || (!disp_scale && !known_type(in_type))) return MOE_A2A_E_DTYPE;
   if (stub_kind != MOE_A2A_STUB_OWNER_RANK && stub_kind != MOE_A2A_STUB_EXPERT_FRACTION) return MOE_A2A_E_DTYPE;
   if (E < 1 || W < 1 || E % W != 0 || R < 0) return MOE_A2A_E_SHAPE;
@@ -1124,7 +1155,7 @@ int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta,
     dim3 grid((unsigned)R * g.nsplit), block(g.threads);
 #define STUB8_LAUNCH(OUT, ST)                                                                                   \
   return launch(KID_STUB_FP8, stub_fp8_kernel<OUT, ST>, grid, block, 0, stream, (const uint2*)disp, disp_scale, meta, \
-                (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit)
+                (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit, rows)
     if (out_type == MOE_A2A_BF16) {
       if (st) STUB8_LAUNCH(Bf16, 1);
       STUB8_LAUNCH(Bf16, 0);
@@ -1140,9 +1171,9 @@ int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta,
   {                                                                                                           \
     if (st)                                                                                                   \
       return launch(KID_STUB, stub_rows_kernel<IN, OUT, 1>, grid, block, 0, stream, (const uint4*)disp, meta, \
-                    (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit);                                     \
+                    (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit, rows);                               \
     return launch(KID_STUB, stub_rows_kernel<IN, OUT, 0>, grid, block, 0, stream, (const uint4*)disp, meta,   \
-                  (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit);                                       \
+                  (uint4*)y, stub_kind, E, E_l, nvec, g.per, g.nsplit, rows);                                 \
   }
   if (in_type == MOE_A2A_BF16 && out_type == MOE_A2A_BF16) STUB_LAUNCH(Bf16, Bf16)
   if (in_type == MOE_A2A_F16 && out_type == MOE_A2A_F16) STUB_LAUNCH(F16, F16)
@@ -1284,10 +1315,10 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
 #undef MOE_A2A_SWITCH_KT
 
 int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
-                    int src_rank, int T, int K, int E, int W, int H, int in_type, int out_type, int fp8_dispatch,
-                    int stub_kind, int combine_mode, int fuse_route, int fuse_stub, int32_t* counts,
-                    int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
-                    void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
+                    int src_rank, int T, int K, int E, int W, int H, int max_recv, int in_type, int out_type,
+                    int fp8_dispatch, int stub_kind, int combine_mode, int fuse_route, int fuse_stub,
+                    int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
+                    int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
                     size_t workspace_bytes, moe_a2a_stream_t stream) {
   if (!known_type(in_type) || !known_type(out_type)) return MOE_A2A_E_DTYPE;
   if (fp8_dispatch && !disp_scale) return MOE_A2A_E_NULL;
@@ -1295,11 +1326,11 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   const bool fused = !fp8_dispatch && (fuse_route == 2 ? (T > 0 && (long long)T * K <= kFusedMaxRows)
                                                          : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
   if (fused) {
-    if (int rc = moe_a2a_route_dispatch(x, indices, rank_start, src_rank, T, K, E, W, H, counts, offsets,
+    if (int rc = moe_a2a_route_dispatch(x, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts, offsets,
                                         slot_of_entry, src_of_slot, meta, status, disp, stream))
       return rc;
   } else {
-    if (int rc = moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, counts, offsets, slot_of_entry,
+    if (int rc = moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
                                src_of_slot, meta, status, workspace, workspace_bytes, stream))
       return rc;
     if (int rc = fp8_dispatch ? moe_a2a_dispatch_fp8(x, in_type, slot_of_entry, (uint8_t*)disp, disp_scale, T, K, H,
@@ -1311,7 +1342,9 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   if (fuse_stub)
     return moe_a2a_stub_combine(disp, scale, indices, weights, slot_of_entry, combine_mode, in_type, out_type,
                                 stub_kind, E, W, out, T, K, H, stream);
-  if (int rc = moe_a2a_stub(disp, scale, meta, in_type, out_type, stub_kind, E, W, expert_y, T * K, H, stream))
+  // padded layout: the stub visits the rows that hold entries, entry by entry
+  if (int rc = moe_a2a_stub(disp, scale, meta, max_recv > 0 ? slot_of_entry : nullptr, in_type, out_type, stub_kind,
+                            E, W, expert_y, T * K, H, stream))
     return rc;
   return moe_a2a_combine(expert_y, weights, slot_of_entry, combine_mode, out_type, out, T, K, H, stream);
 }

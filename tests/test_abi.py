@@ -59,8 +59,10 @@ def test_version_strings_and_queries(lib):
 
 
 def test_route_rejects_bad_arguments(lib):
-    def route(T=4, K=2, E=8, W=2, indices=A, counts=A, offsets=A, soe=A, sos=A, meta=A, ws=A, wsb=1 << 20):
-        return lib.moe_a2a_route(indices, None, 0, T, K, E, W, counts, offsets, soe, sos, meta, None, ws, wsb, None)
+    def route(T=4, K=2, E=8, W=2, indices=A, counts=A, offsets=A, soe=A, sos=A, meta=A, ws=A, wsb=1 << 20,
+              max_recv=0):
+        return lib.moe_a2a_route(indices, None, 0, T, K, E, W, max_recv, counts, offsets, soe, sos, meta, None, ws,
+                                 wsb, None)
 
     assert route(K=0) == E_SHAPE
     assert route(K=33) == E_SHAPE
@@ -70,6 +72,8 @@ def test_route_rejects_bad_arguments(lib):
     assert route(W=0) == E_SHAPE
     assert route(T=-1) == E_SHAPE
     assert route(T=1 << 30, K=8) == E_SHAPE
+    assert route(max_recv=-1) == E_SHAPE
+    assert route(E=1024, W=8, max_recv=1 << 20) == E_SHAPE  # padded rows must stay addressable
     assert route(counts=None) == E_NULL
     assert route(indices=None) == E_NULL
     assert route(meta=None) == E_NULL
@@ -88,10 +92,10 @@ def test_row_functions_reject_bad_arguments(lib):
     assert lib.moe_a2a_dispatch_fp8(A, 7, A, A, A, 4, 2, 128, None) == E_DTYPE
     assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, A, 4, 2, 64, None) == E_SHAPE  # H % 128
     assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, None, 4, 2, 128, None) == E_NULL
-    assert lib.moe_a2a_stub(A, None, A, 5, _lib.BF16, 0, 8, 2, A, 8, 64, None) == E_DTYPE
-    assert lib.moe_a2a_stub(A, None, A, _lib.BF16, _lib.BF16, 9, 8, 2, A, 8, 64, None) == E_DTYPE
-    assert lib.moe_a2a_stub(A, None, A, _lib.BF16, _lib.BF16, 0, 9, 2, A, 8, 64, None) == E_SHAPE
-    assert lib.moe_a2a_stub(A, None, None, _lib.BF16, _lib.BF16, 0, 8, 2, A, 8, 64, None) == E_NULL
+    assert lib.moe_a2a_stub(A, None, A, None, 5, _lib.BF16, 0, 8, 2, A, 8, 64, None) == E_DTYPE
+    assert lib.moe_a2a_stub(A, None, A, None, _lib.BF16, _lib.BF16, 9, 8, 2, A, 8, 64, None) == E_DTYPE
+    assert lib.moe_a2a_stub(A, None, A, None, _lib.BF16, _lib.BF16, 0, 9, 2, A, 8, 64, None) == E_SHAPE
+    assert lib.moe_a2a_stub(A, None, None, None, _lib.BF16, _lib.BF16, 0, 8, 2, A, 8, 64, None) == E_NULL
     assert lib.moe_a2a_combine(A, A, A, 3, _lib.BF16, A, 4, 2, 64, None) == E_DTYPE
     assert lib.moe_a2a_combine(A, A, A, 0, 4, A, 4, 2, 64, None) == E_DTYPE
     assert lib.moe_a2a_combine(A, None, A, 0, _lib.BF16, A, 4, 2, 64, None) == E_NULL
@@ -99,7 +103,7 @@ def test_row_functions_reject_bad_arguments(lib):
     assert lib.moe_a2a_stub_combine(A, None, None, A, A, 0, _lib.BF16, _lib.BF16, 0, 8, 2, A, 4, 2, 64, None) == E_NULL
     assert lib.moe_a2a_stub_combine(A, None, A, A, A, 0, _lib.BF16, _lib.BF16, 0, 8, 3, A, 4, 2, 64, None) == E_SHAPE
     big = lib.moe_a2a_fused_max_rows() // 8 + 1
-    assert lib.moe_a2a_route_dispatch(A, A, None, 0, big, 8, 8, 2, 64, A, A, A, A, A, None, A, None) == E_SHAPE
+    assert lib.moe_a2a_route_dispatch(A, A, None, 0, big, 8, 8, 2, 64, 0, A, A, A, A, A, None, A, None) == E_SHAPE
 
 
 def test_timer_needs_begin_first(lib):

@@ -174,6 +174,60 @@ def test_forward_single_call_equals_separate_calls(gpu_device, name):
                 assert_same("slot_of_entry (planned)", ata.last.slot_of_entry, want["slot_of_entry"])
 
 
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+@pytest.mark.parametrize("fuse_route", ["always", False])
+def test_padded_layout_is_the_reference_dispatch_return_value(gpu_device, name, fuse_route):
+    """padded=True lays the rows out as the reference's [E_l, max_recv, .] buffers: the views
+    handed out per owner rank equal what the reference's own dispatch returned, and the final
+    output is unchanged."""
+    cfg, world, expected = load_golden(name)
+    W = len(world)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, padded=True, fuse_route=fuse_route)
+    d = ata.dispatch(x, idx, rs)
+    ey = ata.expert_stub(d)
+    y = ata.combine(None, w, d, ey)
+    assert int(d.status.item()) == 0
+    E_l = cfg.num_experts // W
+    assert d.disp_x.shape[0] == cfg.num_experts * ata.max_recv and ata.max_recv == cfg.max_num_tokens * W
+    for r, exp in enumerate(expected):
+        num, ex, em = d.padded(r)
+        assert ex.shape == (E_l, ata.max_recv, cfg.hidden_dim) and ex.data_ptr() >= d.disp_x.data_ptr()  # a view
+        assert_same("expert_num_tokens", num, exp.expert_num_tokens)
+        assert_same("expert_x", torch.cat([ex[le, : int(num[le])] for le in range(E_l)], 0), exp.expert_x)
+        assert_same("expert_meta", torch.cat([em[le, : int(num[le])] for le in range(E_l)], 0), exp.expert_meta)
+        ey_r = ey.view(W, E_l, ata.max_recv, cfg.hidden_dim)[r]
+        assert_same("expert_y", torch.cat([ey_r[le, : int(num[le])] for le in range(E_l)], 0), exp.expert_y)
+    assert_same("y", y, golden_compact(cfg, expected)["y"])
+    assert_same("y (single call)", ata.forward(x, idx, w, rs), golden_compact(cfg, expected)["y"])
+
+
+def test_padded_layout_larger_worlds_and_overflow_flag(gpu_device):
+    wl = C.generate_workload("skew_world")
+    want = V.run_world(wl.cfg, wl.world, stub_kind=wl.stub_kind)
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    for fuse_route, max_recv in ((False, 1024), ("always", 1024), (False, None)):
+        ata = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind, padded=True, fuse_route=fuse_route,
+                          max_recv=max_recv)
+        y = ata.forward(x, idx, w, rs)
+        assert_same("y", y, want["y"])
+        d = ata.last
+        assert int(d.status.item()) == 0
+        off = want["offsets"].tolist()
+        rows = d.slot_of_entry.cpu().long()
+        e = idx.flatten().cpu().long()
+        j = want["slot_of_entry"].long() - want["offsets"][e].long()
+        assert torch.equal(rows, e * ata.max_recv + j)  # row = expert * max_recv + position
+        assert_same("rows hold the tokens", d.disp_x[rows.to(gpu_device)], want["disp_x"][want["slot_of_entry"].long()])
+    # the hottest expert receives far more than 64 rows: too small a segment must be flagged
+    for fuse_route in (False, "always"):
+        small = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind, padded=True, max_recv=64,
+                            fuse_route=fuse_route)
+        small.forward(x, idx, w, rs)
+        torch.cuda.synchronize()
+        assert int(small.last.status.item()) == 2
+
+
 def test_custom_kernel_contract(gpu_device):
     """custom_kernel(data) per rank == oracle ref_kernel, checked with the reference's tolerance."""
     from kernel_amd.submission import custom_kernel
