@@ -228,6 +228,51 @@ def test_padded_layout_larger_worlds_and_overflow_flag(gpu_device):
         assert int(small.last.status.item()) == 2
 
 
+@pytest.mark.parametrize("E,K,T,H,W", [(1, 1, 1, 8, 1), (2, 2, 1, 16, 2), (4, 2, 3, 8, 1), (256, 8, 1, 7168, 8),
+                                         (8, 8, 2049, 64, 8)])
+def test_degenerate_shapes(gpu_device, E, K, T, H, W):
+    """One expert, one token, the narrowest rows (a single 16-byte vector), every expert chosen
+    by every token, a table one entry past a tile boundary."""
+    g = torch.Generator().manual_seed(T + H)
+    cfg = C.MoEConfig(E, K, H, T + 1, torch.float16, torch.float16)
+    idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    world = [C.RankData.empty(cfg) for _ in range(W)]
+    world[W - 1] = C.RankData(T, idx, torch.rand(T, K, generator=g), torch.randn(T, H, generator=g).to(torch.float16))
+    for fuse in ("always", False):
+        compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=fuse)
+
+
+def test_unaligned_index_slices_and_out_of_range_ids(gpu_device):
+    """indices / weights that start 4 bytes into an allocation; an expert id outside [0, E) is
+    clamped (nothing is written out of bounds) and raises the status flag."""
+    wl = C.generate_workload("tiny")
+    cfg = wl.cfg
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    T, K = idx.shape
+    idx_store = torch.zeros(T * K + 1, dtype=torch.int32, device=gpu_device)
+    w_store = torch.zeros(T * K + 1, dtype=torch.float32, device=gpu_device)
+    idx_u, w_u = idx_store[1:].view(T, K), w_store[1:].view(T, K)
+    idx_u.copy_(idx)
+    w_u.copy_(w)
+    assert idx_u.data_ptr() % 16 == 4
+    want = V.run_world(cfg, wl.world, stub_kind=1)
+    for fuse in ("always", False):
+        ata = HipAllToAll(cfg, 0, 1, stub_kind=1, fuse_route=fuse)
+        assert_same("y", ata.forward(x, idx_u, w_u), want["y"])
+        assert int(ata.last.status.item()) == 0
+    bad = idx.clone()
+    bad[5, 1] = 99
+    bad[9, 0] = -3
+    clamped = bad.clamp(0, cfg.num_experts - 1)
+    want = V.run_world(cfg, [C.RankData(T, clamped.cpu(), w.cpu(), x.cpu())], stub_kind=1)
+    for fuse in ("always", False):
+        ata = HipAllToAll(cfg, 0, 1, stub_kind=1, fuse_route=fuse)
+        y = ata.forward(x, bad, w)
+        assert int(ata.last.status.item()) == 1
+        assert_same("slot_of_entry", ata.last.slot_of_entry, want["slot_of_entry"])
+        assert_same("disp_x", ata.last.disp_x, want["disp_x"])
+
+
 def test_custom_kernel_contract(gpu_device):
     """custom_kernel(data) per rank == oracle ref_kernel, checked with the reference's tolerance."""
     from kernel_amd.submission import custom_kernel
