@@ -302,18 +302,35 @@ class HipAllToAll:
                           self.max_recv if self.padded else 0)
 
     def forward(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
-                rank_start: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """dispatch -> stub -> combine in one library call; returns ``y[T,H]`` (a buffer the
-        second-next call reuses).  ``self.last`` holds the ``Dispatched`` record of the call."""
+                rank_start: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """dispatch -> stub -> combine in one library call; returns ``y[T,H]``: ``out`` if given
+        (``out_dtype[>=T,H]``, contiguous), else a buffer the second-next call reuses.
+        ``self.last`` holds the ``Dispatched`` record of the call."""
         cfg = self.cfg
-        if x.shape[0] == 0:
+        T = x.shape[0]
+        if T == 0:
             return torch.empty(0, cfg.hidden_dim, dtype=cfg.out_dtype, device=x.device)
         self._check_inputs(x, indices, weights, rank_start)
-        b = self._buffers(x.shape[0], x.device, advance=True)
-        _lib.check(self.lib.moe_a2a_forward(*self._forward_args(b, x, indices, weights, rank_start, _stream())),
-                   "moe_a2a_forward")
-        self.last = self._record(b, x.shape[0])
-        return b["out"]
+        if out is not None:
+            _require_gpu(out, "out")
+            if out.dtype != cfg.out_dtype or out.dim() != 2 or out.shape[0] < T or out.shape[1] != cfg.hidden_dim:
+                raise ValueError("out must be out_dtype[>=T,H]")
+        b = self._buffers(T, x.device, advance=True)
+        # the argument list of a buffer set is built once; a call patches the caller's pointers in
+        args = b.get("_args")
+        if args is None:
+            args = b["_args"] = list(self._forward_args(b, x, indices, weights, rank_start, 0))
+            b["_record"] = self._record(b, T)
+        args[0], args[1], args[2] = x.data_ptr(), indices.data_ptr(), weights.data_ptr()
+        args[3] = None if rank_start is None else rank_start.data_ptr()
+        args[14], args[15] = self.stub_kind, self.combine_mode
+        args[16] = 2 if self.fuse_route == "always" else int(bool(self.fuse_route))
+        args[17] = int(self.fuse_stub)
+        args[27] = b["out"].data_ptr() if out is None else out.data_ptr()
+        args[30] = _stream()
+        _lib.check(self.lib.moe_a2a_forward(*args), "moe_a2a_forward")
+        self.last = b["_record"]
+        return b["out"] if out is None else out
 
     def plan(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
              rank_start: Optional[torch.Tensor] = None, stream: Optional[torch.cuda.Stream] = None):
