@@ -180,6 +180,17 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                     size_t workspace_bytes, moe_a2a_stream_t stream);
 
 /*
+ * Expert compute on the dispatched layout: y[rows of e, :] = x[rows of e, :] * W_e^T for every
+ * expert e, rows of e = [offsets[e], offsets[e+1]) (compact) or [e*max_recv, e*max_recv + count)
+ * (padded).  The reference stands a scalar multiply in for this step (all2all/reference.py:262);
+ * this is the grouped matrix product a real MoE layer runs there.
+ *   x[rows, Kd], weights[E, N, Kd], y[rows, N]: 16-bit elements of elem_type, f32 accumulation,
+ *   Kd % 64 == 0, N % 8 == 0, 16-byte aligned.
+ */
+int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offsets, void* y, int R, int E, int Kd,
+                        int N, int max_recv, int elem_type, moe_a2a_stream_t stream);
+
+/*
  * Launch timer (opt-in, process-wide, single caller thread).  Between begin and end every
  * kernel the library launches carries a pair of HIP events bound to that dispatch, so the
  * reported time is the kernel's own begin-to-end duration on the GPU.

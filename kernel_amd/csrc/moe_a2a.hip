@@ -43,11 +43,12 @@ enum KernelId {
   KID_STUB_FP8,
   KID_COMBINE,
   KID_STUB_COMBINE,
+  KID_EXPERT_GEMM,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch",
-    "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine"};
+    "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -922,6 +923,164 @@ __global__ __launch_bounds__(kRowMaxThreads) void stub_combine_fp8_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// expert compute: grouped GEMM over the expert segments (the step between dispatch and combine)
+// ---------------------------------------------------------------------------------------
+// y[rows of e, :] = x[rows of e, :] * W_e^T with W_e[N, Kd] (both operands K-contiguous), f32
+// accumulation on the matrix cores (v_mfma_f32_32x32x16), one rounding to the 16-bit output.
+// A workgroup of four waves owns a 128x128 output tile (each wave 64x64 = 2x2 MFMA blocks);
+// K advances 64 at a time through LDS (row stride 72 elements, so the 16-byte fragment reads
+// of 16 consecutive rows fall on disjoint banks); the next K slab is fetched into registers
+// while the current one is multiplied.  Tiles are numbered n-fastest, so with N/128 a multiple
+// of 8 every m-tile that needs the weight slab (e, n-tile) runs on the same XCD and finds it in
+// that XCD's L2.
+constexpr int kGemmM = 128, kGemmN = 128, kGemmK = 64;
+constexpr int kGemmLd = kGemmK + 8;  // LDS row stride in elements
+constexpr int kGemmThreads = 256;
+
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+
+template <class E>
+__device__ __forceinline__ f32x16_t mfma_32x32x16(const uint4& a, const uint4& b, const f32x16_t& c);
+template <>
+__device__ __forceinline__ f32x16_t mfma_32x32x16<Bf16>(const uint4& a, const uint4& b, const f32x16_t& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16_t mfma_32x32x16<F16>(const uint4& a, const uint4& b, const f32x16_t& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                0, 0);
+}
+
+template <class E>
+__global__ __launch_bounds__(kGemmThreads) void expert_gemm_kernel(const uint4* __restrict__ x,
+                                                                    const uint4* __restrict__ w,
+                                                                    const int32_t* __restrict__ offsets,
+                                                                    uint16_t* __restrict__ y, int num_experts,
+                                                                    int Kd, int N, int max_recv, int ntile_n) {
+  __shared__ __attribute__((aligned(16))) uint16_t s_ab[(kGemmM + kGemmN) * kGemmLd];
+  uint16_t* s_a = s_ab;
+  uint16_t* s_b = s_ab + kGemmM * kGemmLd;
+  __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
+  __shared__ int s_tmp[kGemmThreads / kWave + 1];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+
+  // which (expert, m-tile, n-tile) is this workgroup?  m-tiles of all experts are numbered in
+  // expert order; the prefix of ceil(count/128) is scanned here (E <= 1024: four per thread)
+  const int tile_n = blockIdx.x % ntile_n;
+  const int tile_m_global = blockIdx.x / ntile_n;
+  {
+    const int span = (num_experts + kGemmThreads - 1) / kGemmThreads;
+    const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += (offsets[e + 1] - offsets[e] + kGemmM - 1) / kGemmM;
+    int total;
+    int run = block_exclusive_scan(sum, s_tmp, total);
+    for (int e = lo; e < hi; ++e) {
+      s_pref[e] = run;
+      run += (offsets[e + 1] - offsets[e] + kGemmM - 1) / kGemmM;
+    }
+    if (tid == 0) s_pref[num_experts] = total;
+    __syncthreads();
+    if (tile_m_global >= total) return;  // the grid is sized for the worst case
+  }
+  int e_lo = 0, e_hi = num_experts;  // largest e with s_pref[e] <= tile_m_global
+  while (e_hi - e_lo > 1) {
+    int mid = (e_lo + e_hi) >> 1;
+    if (s_pref[mid] <= tile_m_global) e_lo = mid; else e_hi = mid;
+  }
+  const int e = e_lo;
+  const int count = offsets[e + 1] - offsets[e];
+  const int m0 = (tile_m_global - s_pref[e]) * kGemmM;          // first row of the tile inside the segment
+  const size_t row0 = (size_t)(max_recv > 0 ? e * max_recv : offsets[e]) + m0;  // its row in x and y
+  const int rows = min(kGemmM, count - m0);
+  const int n0 = tile_n * kGemmN;
+  const int kvec = Kd / 8;  // 16-byte vectors per row
+
+  // global -> register prefetch: a 128 x 64 slab is 1024 vectors, four per thread (8 per row)
+  const uint4* xa = x + row0 * kvec;
+  const uint4* wb = w + ((size_t)e * N + n0) * kvec;
+  uint4 ra[4], rb[4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int v = tid + i * kGemmThreads;
+      const int r = v >> 3, c = v & 7;
+      ra[i] = r < rows ? xa[(size_t)r * kvec + (k0 >> 3) + c] : make_uint4(0, 0, 0, 0);
+      rb[i] = n0 + r < N ? wb[(size_t)r * kvec + (k0 >> 3) + c] : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int v = tid + i * kGemmThreads;
+      const int r = v >> 3, c = v & 7;
+      *reinterpret_cast<uint4*>(&s_a[r * kGemmLd + c * 8]) = ra[i];
+      *reinterpret_cast<uint4*>(&s_b[r * kGemmLd + c * 8]) = rb[i];
+    }
+  };
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;  // this wave's 64x64 corner of the tile
+  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+
+  fetch(0);
+  for (int k0 = 0; k0 < Kd; k0 += kGemmK) {
+    stash();
+    __syncthreads();
+    if (k0 + kGemmK < Kd) fetch(k0 + kGemmK);  // in flight during the multiplies below
+#pragma unroll
+    for (int kk = 0; kk < kGemmK; kk += 16) {
+      uint4 fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa[i] = *reinterpret_cast<const uint4*>(&s_a[(wm + i * 32 + frag_row) * kGemmLd + kk + frag_k]);
+        fb[i] = *reinterpret_cast<const uint4*>(&s_b[(wn + i * 32 + frag_row) * kGemmLd + kk + frag_k]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x16<E>(fa[i], fb[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: round to the output type into LDS (the tile is 128 x 128 x 2 B = 32 KB, the operand
+  // buffer holds 36 KB), then 16-byte row stores.  Accumulator element q of a
+  // 32x32 block sits at row (q/4)*8 + (lane/32)*4 + q%4, column lane%32.
+  uint16_t* s_c = s_ab;
+  constexpr int kCLd = kGemmN + 8;
+  static_assert(kGemmM * kCLd <= (kGemmM + kGemmN) * kGemmLd, "output tile must fit the operand buffer");
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int r = wm + i * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
+        const int c = wn + j * 32 + (lane & 31);
+        s_c[r * kCLd + c] = (uint16_t)(E::pack(acc[i][j][q], 0.f) & 0xffffu);
+      }
+  __syncthreads();
+  for (int v = tid; v < kGemmM * (kGemmN / 8); v += kGemmThreads) {
+    const int r = v / (kGemmN / 8), c = (v % (kGemmN / 8)) * 8;
+    if (r < rows && n0 + c < N)
+      *reinterpret_cast<uint4*>(y + (row0 + r) * (size_t)N + n0 + c) = *reinterpret_cast<const uint4*>(&s_c[r * kCLd + c]);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
 struct LaunchTimer {
@@ -1347,6 +1506,28 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                             E, W, expert_y, T * K, H, stream))
     return rc;
   return moe_a2a_combine(expert_y, weights, slot_of_entry, combine_mode, out_type, out, T, K, H, stream);
+}
+
+int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offsets, void* y, int R, int E, int Kd,
+                        int N, int max_recv, int elem_type, moe_a2a_stream_t stream_) {
+  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
+  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < kGemmK || Kd % kGemmK != 0 || N < 8 || N % 8 != 0 ||
+      max_recv < 0)
+    return MOE_A2A_E_SHAPE;
+  if (R == 0) return 0;
+  if (!x || !weights || !offsets || !y) return MOE_A2A_E_NULL;
+  if (!aligned16(x) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
+  const int ntile_n = ceil_div(N, kGemmN);
+  // worst case of m-tiles: every expert ends with a partly filled tile
+  const long long mtiles = (long long)R / kGemmM + E;
+  if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
+  dim3 grid((unsigned)(mtiles * ntile_n)), block(kGemmThreads);
+  hipStream_t stream = (hipStream_t)stream_;
+  if (elem_type == MOE_A2A_BF16)
+    return launch(KID_EXPERT_GEMM, expert_gemm_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
+                  (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+  return launch(KID_EXPERT_GEMM, expert_gemm_kernel<F16>, grid, block, 0, stream, (const uint4*)x,
+                (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
 }
 
 int moe_a2a_timer_begin(int capacity) {

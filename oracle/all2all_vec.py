@@ -129,6 +129,21 @@ def stub(disp_x: torch.Tensor, meta: torch.Tensor, stub_kind: int, num_experts: 
     return (disp_x.to(out_dtype).to(torch.float32) * s).to(out_dtype)
 
 
+def expert_gemm(disp_x: torch.Tensor, offsets: torch.Tensor, weights: torch.Tensor,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-expert linear layer on the compact rows: ``y[seg e] = x[seg e] @ W_e^T`` computed in f32
+    and rounded once.  Has no counterpart in the reference (its expert is the scalar stub); the
+    HIP kernel is compared with this within a tolerance, because the summation order differs."""
+    R = disp_x.shape[0]
+    E, N, _ = weights.shape
+    y = torch.zeros(R, N, dtype=out_dtype)
+    off = offsets.tolist()
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            y[off[e]:off[e + 1]] = (disp_x[off[e]:off[e + 1]].float() @ weights[e].float().t()).to(out_dtype)
+    return y
+
+
 def combine_strict(expert_y: torch.Tensor, weights: torch.Tensor, slot_of_entry: torch.Tensor,
                    out_dtype: torch.dtype) -> torch.Tensor:
     """Reference-order weighted sum with a rounding to ``out_dtype`` after every add."""

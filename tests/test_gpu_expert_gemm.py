@@ -1,0 +1,87 @@
+"""Grouped expert GEMM (matrix cores) against an f32 torch reference of the same product.
+
+The summation order differs from torch's, so the comparison is a tolerance, stated here:
+|got - want| <= 1e-2 * |want| + 1e-2 * rms(want) (one bf16 ulp is 0.4-0.8 %; fp16 is tighter).
+"""
+import pytest
+import torch
+
+from kernel_amd import contract as C
+from kernel_amd.all2all import HipAllToAll, concat_world
+from oracle import all2all_vec as V
+
+pytestmark = pytest.mark.gpu
+
+
+def close(got, want):
+    got, want = got.float().cpu(), want.float()
+    tol = 1e-2 * want.abs() + 1e-2 * want.pow(2).mean().sqrt()
+    bad = (got - want).abs() > tol
+    assert not bool(bad.any()), f"{int(bad.sum())} of {bad.numel()} out of tolerance, worst " \
+                                f"{float(((got - want).abs() / tol).max()):.2f}x"
+
+
+def make(E, K, T, H, N, W, dtype, seed, zipf=False):
+    g = torch.Generator().manual_seed(seed)
+    cfg = C.MoEConfig(E, K, H, T + 1, dtype, dtype)
+    if zipf:
+        p = (torch.arange(E, dtype=torch.float64) + 1).pow(-1.2)
+        idx = torch.multinomial((p / p.sum()).float().expand(T, E), K, generator=g).to(torch.int32)
+    else:
+        idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    world = [C.RankData(T, idx, torch.rand(T, K, generator=g), torch.randn(T, H, generator=g).to(dtype))]
+    world += [C.RankData.empty(cfg) for _ in range(W - 1)]
+    weights = (torch.randn(E, N, H, generator=g) / H ** 0.5).to(dtype)
+    return cfg, world, weights
+
+
+@pytest.mark.parametrize("E,K,T,H,N,W,zipf", [
+    (8, 2, 40, 64, 64, 1, False),      # one K slab, tiles mostly empty
+    (8, 2, 700, 128, 200, 2, False),   # several m-tiles per expert, N not a multiple of 128
+    (16, 4, 300, 192, 136, 4, True),   # skewed: empty experts and long segments
+    (64, 6, 1024, 2048, 2048, 8, True),
+    (256, 8, 256, 7168, 512, 8, False),  # headline routing shape, 8 rows per expert on average
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
+def test_expert_gemm_matches_f32_reference(gpu_device, E, K, T, H, N, W, zipf, dtype, padded):
+    cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=E + T, zipf=zipf)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, padded=padded, max_recv=T if padded else None)
+    d = ata.dispatch(x, idx, rs)
+    y = ata.expert_gemm(d, weights.to(gpu_device))
+    torch.cuda.synchronize()
+    o = V.run_world(cfg, world)
+    want = V.expert_gemm(o["disp_x"], o["offsets"], weights, dtype)
+    rows = d.slot_of_entry.long() if padded else o["slot_of_entry"].long().to(gpu_device)
+    close(y[rows], want[o["slot_of_entry"].long()])
+    if not padded:
+        close(y, want)
+
+
+def test_dispatch_gemm_combine_end_to_end(gpu_device):
+    """dispatch -> expert GEMM (H -> H) -> combine against the same chain on the CPU."""
+    cfg, world, weights = make(32, 4, 512, 256, 256, 8, torch.bfloat16, seed=3)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, 8, combine_mode=C.COMBINE_F32)
+    d = ata.dispatch(x, idx, rs)
+    y = ata.combine(None, w, d, ata.expert_gemm(d, weights.to(gpu_device)))
+    o = V.run_world(cfg, world)
+    ey = V.expert_gemm(o["disp_x"], o["offsets"], weights, torch.bfloat16)
+    want = V.combine_f32(ey, w.cpu(), o["slot_of_entry"], torch.bfloat16)
+    close(y, want)
+
+
+def test_expert_gemm_argument_checks(gpu_device):
+    cfg, world, weights = make(8, 2, 16, 64, 64, 1, torch.bfloat16, seed=1)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, 1)
+    d = ata.dispatch(x, idx)
+    with pytest.raises(ValueError):
+        ata.expert_gemm(d, weights[:, :, :32].contiguous().to(gpu_device))
+    bad = HipAllToAll(C.MoEConfig(8, 2, 72, 17, torch.bfloat16, torch.bfloat16), 0, 1)
+    xb = torch.randn(16, 72, device=gpu_device).to(torch.bfloat16)
+    db = bad.dispatch(xb, idx)
+    from kernel_amd._lib import MoeA2AError
+    with pytest.raises(MoeA2AError):  # hidden size must be a multiple of 64
+        bad.expert_gemm(db, torch.zeros(8, 64, 72, dtype=torch.bfloat16, device=gpu_device))
