@@ -59,6 +59,9 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--cold", action="store_true", help="add a leg with caches flushed before every step")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
+    p.add_argument("--expert-gemm", type=int, default=0, metavar="N",
+                   help="measure the grouped expert GEMM (N output columns per expert) on the workload's "
+                        "dispatched rows instead of the dispatch/combine path")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="end with three plain 256 MiB device copies (a known-size reference for rocprof counters)")
     return p.parse_args()
@@ -154,6 +157,8 @@ def main():
     ata = HipAllToAll(cfg, 0, W, stub_kind=wl.stub_kind, combine_mode=mode, fp8_dispatch=fp8,
                       fuse_route=not args.no_fuse_route, fuse_stub=args.fuse_stub)
     x, idx, w, rs = concat_world(wl.world, dev)
+    if args.expert_gemm:
+        return expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev)
 
     # Everything runs on one non-blocking stream of its own: launches on the legacy default
     # stream carry implicit waits on every other stream of the process.
@@ -276,6 +281,77 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(wl, mode, fp8, y, b_dc, args.cpu_seconds)
     print(json.dumps(out, ensure_ascii=False), flush=True)
+
+
+MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16
+
+
+def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
+    """Grouped expert GEMM y[seg e] = x[seg e] @ W_e^T on the workload's 16-bit dispatched rows.
+    One JSON line: TFLOP/s against the dense 16-bit MFMA peak, kernel time from the launch timer,
+    and a CPU leg (the oracle's per-expert f32 matmul on a bounded number of experts) that also
+    checks the GPU rows it covers."""
+    from kernel_amd.all2all import HipAllToAll
+
+    cfg = wl.cfg
+    E, H, N = cfg.num_experts, cfg.hidden_dim, args.expert_gemm
+    ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind)
+    gen = torch.Generator(device="cpu").manual_seed(1234)
+    weights = (torch.randn(E, N, H, generator=gen) / H ** 0.5).to(cfg.in_dtype).to(dev)
+    main = torch.cuda.Stream()
+    main.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(main):
+        d = ata.dispatch(x, idx, rs)
+        R = d.num_rows
+        y = torch.empty(R, N, dtype=cfg.in_dtype, device=dev)
+        for _ in range(args.warmup):
+            ata.expert_gemm(d, weights, out=y)
+        main.synchronize()
+        per = kernel_times(lib, lambda n: [ata.expert_gemm(d, weights, out=y) for _ in range(n)], args.steps, torch)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(main)
+        for _ in range(args.steps):
+            ata.expert_gemm(d, weights, out=y)
+        e1.record(main)
+        main.synchronize()
+    ms_step = e0.elapsed_time(e1) / args.steps
+    t_us = statistics.fmean(per["expert_gemm"])
+    flops = 2.0 * R * H * N
+    tflops = flops / t_us / 1e6
+    out = dict(metric=f"grouped expert GEMM TFLOP/s, {E}E h{H} n{N} bf16", value=round(tflops, 1), unit="TFLOP/s",
+               n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 5), higher_is_better=True,
+               scaling="weak", vs_baseline=None, dtype="bf16" if cfg.in_dtype == torch.bfloat16 else "f16",
+               data="synthetic",
+               config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N),
+               kernels_us=summarise(per),
+               roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                             frac=round(tflops / MFMA_PEAK_TFLOPS, 4), traffic=None))
+    if not args.no_cpu:
+        from oracle import all2all_vec as O
+
+        off = d.offsets.cpu()
+        dx, wc, yg = d.disp_x.cpu(), weights.cpu(), y.cpu()
+        t0, done, rows_done, worst = time.perf_counter(), 0, 0, 0.0
+        for e in range(E):
+            lo, hi = int(off[e]), int(off[e + 1])
+            if hi > lo:
+                ref = O.expert_gemm(dx[lo:hi], torch.tensor([0, hi - lo], dtype=torch.int32), wc[e:e + 1], cfg.in_dtype)
+                want, got = ref.float(), yg[lo:hi].float()
+                # summation order differs from the CPU's: 1 % of the value + 1 % of the segment's rms
+                tol = 1e-2 * want.abs() + 1e-2 * want.pow(2).mean().sqrt()
+                worst = max(worst, float(((got - want).abs() / tol).max()))
+                rows_done += hi - lo
+            done += 1
+            if time.perf_counter() - t0 > args.cpu_seconds:
+                break
+        dt = time.perf_counter() - t0
+        if worst > 1.0:
+            raise RuntimeError(f"expert GEMM outside the tolerance of the f32 reference: {worst:.2f}x")
+        out["cpu_baseline"] = dict(value=round(2.0 * rows_done * H * N / dt / 1e12, 4), unit="TFLOP/s",
+                                   cores=torch.get_num_threads(), kind="port",
+                                   sample=f"first {done} of {E} experts ({rows_done} rows), f32 matmul; "
+                                          f"worst error {worst:.2f} of the tolerance")
+    print(json.dumps(out))
 
 
 def cpu_baseline(wl, mode, fp8, y_gpu, b_dc, budget_s):
