@@ -315,14 +315,15 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
         e1.record(main)
         main.synchronize()
     ms_step = e0.elapsed_time(e1) / args.steps
-    t_us = statistics.fmean(per["expert_gemm"])
+    kernel = "expert_gemm_wide" if "expert_gemm_wide" in per else "expert_gemm"
+    t_us = statistics.fmean(per[kernel])
     flops = 2.0 * R * H * N
     tflops = flops / t_us / 1e6
     out = dict(metric=f"grouped expert GEMM TFLOP/s, {E}E h{H} n{N} bf16", value=round(tflops, 1), unit="TFLOP/s",
                n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 5), higher_is_better=True,
                scaling="weak", vs_baseline=None, dtype="bf16" if cfg.in_dtype == torch.bfloat16 else "f16",
                data="synthetic",
-               config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N),
+               config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N, kernel=kernel),
                kernels_us=summarise(per),
                roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
                              frac=round(tflops / MFMA_PEAK_TFLOPS, 4), traffic=None))

@@ -15,6 +15,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "moe_a2a.h"
 
@@ -44,11 +45,13 @@ enum KernelId {
   KID_COMBINE,
   KID_STUB_COMBINE,
   KID_EXPERT_GEMM,
+  KID_EXPERT_GEMM_WIDE,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch",
-    "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm"};
+    "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
+    "expert_gemm_wide"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -1074,6 +1077,217 @@ __global__ __launch_bounds__(kGemmThreads) void expert_gemm_kernel(const uint4* 
       }
 }
 
+// Wide variant for long segments: 256 x 256 output tile, four waves of 128 x 128 (a 4 x 4 grid of
+// 32x32 accumulator blocks, 256 AGPRs), K slabs of 64.  One wave per SIMD and one workgroup per
+// CU, so latency is hidden inside the wave: operand slabs are double-buffered in LDS (144 KB),
+// the next slab travels global -> registers a whole iteration ahead, and the fragments of step
+// kk+1 are read from LDS while the sixteen MFMAs of step kk issue.  Per output element a wave
+// reads half the LDS bytes of the 128 x 128 kernel, which is what bounds that kernel (one
+// ds_read_b128 per MFMA at 128 B/clk per CU).  The scheduling-group barriers pin the interleave;
+// the scheduling barriers keep the compiler from sinking a step's fragment reads into the next
+// step, where they would be waited on at once.  Accumulation order over K equals the 128 x 128
+// kernel's, so both give the same bits.
+constexpr int kWideM = 256, kWideN = 256, kWideK = 64, kWideLd = kWideK + 8, kWideThreads = 256;
+constexpr size_t kWideLdsBytes = 2 * (size_t)(kWideM + kWideN) * kWideLd * sizeof(uint16_t);
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+template <class E>
+__device__ __forceinline__ f32x16_t mfma_32x32x16_v(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c);
+template <>
+__device__ __forceinline__ f32x16_t mfma_32x32x16_v<Bf16>(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16_t mfma_32x32x16_v<F16>(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                0, 0);
+}
+
+template <class E>
+__global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const uint4* __restrict__ x,
+                                                                         const uint4* __restrict__ w,
+                                                                         const int32_t* __restrict__ offsets,
+                                                                         uint16_t* __restrict__ y, int num_experts,
+                                                                         int Kd, int N, int max_recv, int ntile_n) {
+  constexpr int TM = kWideM, TN = kWideN, BK = kWideK, LD = kWideLd, NT = kWideThreads;
+  extern __shared__ __attribute__((aligned(16))) uint16_t s_wide[];  // [2][TM + TN][LD]
+  __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
+  __shared__ int s_tmp[NT / kWave + 1];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+
+  // (expert, m-tile, n-tile) of this workgroup, as in the 128 x 128 kernel with 256-row tiles
+  const int tile_n = blockIdx.x % ntile_n;
+  const int tile_m_global = blockIdx.x / ntile_n;
+  {
+    const int span = (num_experts + NT - 1) / NT;
+    const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    int total;
+    int run = block_exclusive_scan(sum, s_tmp, total);
+    for (int e = lo; e < hi; ++e) {
+      s_pref[e] = run;
+      run += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    }
+    if (tid == 0) s_pref[num_experts] = total;
+    __syncthreads();
+    if (tile_m_global >= total) return;
+  }
+  int e_lo = 0, e_hi = num_experts;
+  while (e_hi - e_lo > 1) {
+    int mid = (e_lo + e_hi) >> 1;
+    if (s_pref[mid] <= tile_m_global) e_lo = mid; else e_hi = mid;
+  }
+  const int e = e_lo;
+  const int count = offsets[e + 1] - offsets[e];
+  const int m0 = (tile_m_global - s_pref[e]) * TM;
+  const size_t row0 = (size_t)(max_recv > 0 ? e * max_recv : offsets[e]) + m0;
+  const int rows = min(TM, count - m0);
+  const int n0 = tile_n * TN;
+  const int ncols = min(TN, N - n0);
+  const int kvec = Kd / 8;
+  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * kvec;
+  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * kvec;
+
+  // A slab is 256 rows x 8 vectors for each operand: eight vectors of each per thread.  Rows past
+  // the segment and columns past N read the last valid row instead of zeros: they only feed
+  // accumulators that are never stored, and the loads stay unconditional.
+  constexpr int VPR = BK / 8, NA = TM * VPR / NT, NB = TN * VPR / NT;
+  int offa[NA], offb[NB];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int v = tid + i * NT;
+    offa[i] = min(v / VPR, rows - 1) * kvec + v % VPR;
+  }
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int v = tid + i * NT;
+    offb[i] = min(v / VPR, ncols - 1) * kvec + v % VPR;
+  }
+  // native vectors, not uint4: the struct type keeps the staging arrays in scratch memory
+  u32x4_t ra[NA], rb[NB];
+  const int st_off = (tid / VPR) * LD + (tid % VPR) * 8;
+#define WIDE_FETCH(K0)                                                           \
+  {                                                                              \
+    const int kv_ = (K0) >> 3;                                                   \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i) ra[i] = xa[offa[i] + kv_];    \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) rb[i] = wb[offb[i] + kv_];    \
+  }
+#define WIDE_STASH(BUF)                                                                                        \
+  {                                                                                                            \
+    uint16_t* s_a_ = s_wide + (BUF) * (TM + TN) * LD + st_off;                                                 \
+    uint16_t* s_b_ = s_a_ + TM * LD;                                                                           \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i)                                                             \
+        *reinterpret_cast<u32x4_t*>(&s_a_[i * (NT / VPR) * LD]) = ra[i];                                       \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                             \
+        *reinterpret_cast<u32x4_t*>(&s_b_[i * (NT / VPR) * LD]) = rb[i];                                       \
+  }
+
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+  const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+  const int fr_a = (wm + (lane & 31)) * LD + (lane >> 5) * 8;
+  const int fr_b = (TM + wn + (lane & 31)) * LD + (lane >> 5) * 8;
+  u32x4_t f0a[4], f0b[4], f1a[4], f1b[4];
+#define WIDE_FRAGS(FA, FB, BUF, KK)                                                                            \
+  {                                                                                                            \
+    const uint16_t* base_ = s_wide + (BUF) * (TM + TN) * LD + (KK);                                            \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                              \
+        FA[i] = *reinterpret_cast<const u32x4_t*>(&base_[fr_a + i * 32 * LD]);                                 \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                              \
+        FB[j] = *reinterpret_cast<const u32x4_t*>(&base_[fr_b + j * 32 * LD]);                                 \
+  }
+#define WIDE_MMA(FA, FB)                                                                                       \
+  {                                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                              \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16_v<E>(FA[i], FB[j], acc[i][j]);     \
+  }
+  // instruction classes of the scheduling groups: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read, 0x200 LDS write
+#define WIDE_MIX_READS() /* 8 x (LDS read, MFMA), then the other 8 MFMAs */                                     \
+  {                                                                                                            \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       \
+    }                                                                                                          \
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);                                                         \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
+  }
+#define WIDE_MIX_WRITES() /* the 8 LDS reads, then 8 x (2 MFMA, 2 LDS writes) */                                \
+  {                                                                                                            \
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);                                                         \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);                                                       \
+    }                                                                                                          \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
+  }
+#define WIDE_MIX_FETCH() /* 8 x (LDS read, MFMA, global load), then 8 x (MFMA, global load) */                  \
+  {                                                                                                            \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                       \
+    }                                                                                                          \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                       \
+    }                                                                                                          \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
+  }
+
+  // The prefetches past the last slab re-read the last slab (clamped k) and land in a buffer
+  // nobody reads: the loop body stays free of branches.
+  WIDE_FETCH(0);
+  WIDE_STASH(0);
+  WIDE_FETCH(min(BK, Kd - BK));
+  __syncthreads();
+  WIDE_FRAGS(f0a, f0b, 0, 0);
+  int buf = 0;
+  for (int k0 = 0; k0 < Kd; k0 += BK, buf ^= 1) {
+    WIDE_FRAGS(f1a, f1b, buf, 16);
+    WIDE_MMA(f0a, f0b);
+    WIDE_MIX_READS();
+    __syncthreads();  // every wave has left the previous slab: the other buffer is free
+    WIDE_FRAGS(f0a, f0b, buf, 32);
+    WIDE_STASH(buf ^ 1);
+    WIDE_MMA(f1a, f1b);
+    WIDE_MIX_WRITES();
+    WIDE_FETCH(min(k0 + 2 * BK, Kd - BK));
+    WIDE_FRAGS(f1a, f1b, buf, 48);
+    WIDE_MMA(f0a, f0b);
+    WIDE_MIX_FETCH();
+    __syncthreads();  // the other buffer is complete
+    WIDE_FRAGS(f0a, f0b, buf ^ 1, 0);
+    WIDE_MMA(f1a, f1b);
+    WIDE_MIX_READS();
+  }
+#undef WIDE_FETCH
+#undef WIDE_STASH
+#undef WIDE_FRAGS
+#undef WIDE_MMA
+#undef WIDE_MIX_READS
+#undef WIDE_MIX_WRITES
+#undef WIDE_MIX_FETCH
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int r = wm + i * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
+        const int c = wn + j * 32 + (lane & 31);
+        if (r < rows && c < ncols)
+          y[(row0 + r) * (size_t)N + n0 + c] = (uint16_t)(E::pack(acc[i][j][q], 0.f) & 0xffffu);
+      }
+}
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -1511,12 +1725,36 @@ int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offse
   if (R == 0) return 0;
   if (!x || !weights || !offsets || !y) return MOE_A2A_E_NULL;
   if (!aligned16(x) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
+  hipStream_t stream = (hipStream_t)stream_;
+  // Long segments take the 256 x 256 kernel: with fewer than 256 rows per expert on average most
+  // of its tiles would be half empty.  MOE_A2A_GEMM_TILE=128|256 in the environment overrides.
+  bool wide = (long long)R >= 256ll * E && N >= kWideN;
+  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) wide = atoi(forced) == 256;
+  if (wide) {
+    const int ntile_n = ceil_div(N, kWideN);
+    const long long mtiles = (long long)R / kWideM + E;  // every expert may end with a partly filled tile
+    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
+    dim3 grid((unsigned)(mtiles * ntile_n)), block(kWideThreads);
+    static bool lds_raised = false;  // the kernels need more dynamic LDS than the 64 KB default
+    if (!lds_raised) {
+      hipError_t e1 = hipFuncSetAttribute((const void*)expert_gemm_wide_kernel<Bf16>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
+      hipError_t e2 = hipFuncSetAttribute((const void*)expert_gemm_wide_kernel<F16>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
+      if (e1 != hipSuccess || e2 != hipSuccess) return (int)(e1 != hipSuccess ? e1 : e2);
+      lds_raised = true;
+    }
+    if (elem_type == MOE_A2A_BF16)
+      return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<Bf16>, grid, block, kWideLdsBytes, stream,
+                    (const uint4*)x, (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+    return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<F16>, grid, block, kWideLdsBytes, stream,
+                  (const uint4*)x, (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+  }
   const int ntile_n = ceil_div(N, kGemmN);
   // worst case of m-tiles: every expert ends with a partly filled tile
   const long long mtiles = (long long)R / kGemmM + E;
   if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
   dim3 grid((unsigned)(mtiles * ntile_n)), block(kGemmThreads);
-  hipStream_t stream = (hipStream_t)stream_;
   if (elem_type == MOE_A2A_BF16)
     return launch(KID_EXPERT_GEMM, expert_gemm_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
                   (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);

@@ -44,7 +44,9 @@ def make(E, K, T, H, N, W, dtype, seed, zipf=False):
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-def test_expert_gemm_matches_f32_reference(gpu_device, E, K, T, H, N, W, zipf, dtype, padded):
+@pytest.mark.parametrize("tile", ["128", "256"], ids=["tile128", "tile256"])
+def test_expert_gemm_matches_f32_reference(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, padded, tile):
+    monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile)  # both kernels on every shape
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=E + T, zipf=zipf)
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, W, padded=padded, max_recv=T if padded else None)
@@ -57,6 +59,40 @@ def test_expert_gemm_matches_f32_reference(gpu_device, E, K, T, H, N, W, zipf, d
     close(y[rows], want[o["slot_of_entry"].long()])
     if not padded:
         close(y, want)
+
+
+@pytest.mark.parametrize("E,K,T,H,N,zipf", [
+    (8, 2, 1200, 192, 264, False),   # 300 rows per expert: the library itself picks the 256 x 256 kernel
+    (16, 4, 1500, 256, 512, True),   # skewed, segments from empty to well past one tile
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_both_tile_sizes_give_the_same_bits(gpu_device, monkeypatch, E, K, T, H, N, zipf, dtype):
+    """The two kernels accumulate over K in the same order, so their outputs are identical; the
+    default choice for these shapes (R >= 256 E) is the wide one."""
+    cfg, world, weights = make(E, K, T, H, N, 1, dtype, seed=7 * E + T, zipf=zipf)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, 1)
+    d = ata.dispatch(x, idx, rs)
+    wd = weights.to(gpu_device)
+    lib = ata.lib
+    outs = {}
+    for tile in ("default", "128", "256"):
+        if tile == "default":
+            monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
+        else:
+            monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile)
+        assert lib.moe_a2a_timer_begin(4) == 0
+        outs[tile] = ata.expert_gemm(d, wd).clone()
+        torch.cuda.synchronize()
+        import ctypes
+        ids, us = (ctypes.c_int * 4)(), (ctypes.c_float * 4)()
+        assert lib.moe_a2a_timer_end(ids, us, 4) == 1
+        name = lib.moe_a2a_kernel_name(ids[0]).decode()
+        assert name == ("expert_gemm" if tile == "128" else "expert_gemm_wide")
+    assert torch.equal(outs["128"].view(torch.int16), outs["256"].view(torch.int16))
+    assert torch.equal(outs["default"].view(torch.int16), outs["256"].view(torch.int16))
+    o = V.run_world(cfg, world)
+    close(outs["256"], V.expert_gemm(o["disp_x"], o["offsets"], weights, dtype))
 
 
 def test_dispatch_gemm_combine_end_to_end(gpu_device):
