@@ -1086,7 +1086,8 @@ __global__ __launch_bounds__(kGemmThreads) void expert_gemm_kernel(const uint4* 
 // ds_read_b128 per MFMA at 128 B/clk per CU).  The scheduling-group barriers pin the interleave;
 // the scheduling barriers keep the compiler from sinking a step's fragment reads into the next
 // step, where they would be waited on at once.  Accumulation order over K equals the 128 x 128
-// kernel's, so both give the same bits.
+// kernel's, so both give the same bits.  Tiles with at most 128 rows take a 128 x 256 form of the
+// same loop.
 constexpr int kWideM = 256, kWideN = 256, kWideK = 64, kWideLd = kWideK + 8, kWideThreads = 256;
 constexpr size_t kWideLdsBytes = 2 * (size_t)(kWideM + kWideN) * kWideLd * sizeof(uint16_t);
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
@@ -1104,56 +1105,22 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16_v<F16>(const u32x4_t& a, const
                                                 0, 0);
 }
 
-template <class E>
-__global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const uint4* __restrict__ x,
-                                                                         const uint4* __restrict__ w,
-                                                                         const int32_t* __restrict__ offsets,
-                                                                         uint16_t* __restrict__ y, int num_experts,
-                                                                         int Kd, int N, int max_recv, int ntile_n) {
+constexpr int wide_gcd(int a, int b) { return b == 0 ? a : wide_gcd(b, a % b); }
+
+// Main loop and epilogue of one wide tile.  Each wave owns WMI x WNJ accumulator blocks of 32 x 32
+// at (wm, wn); AROWS rows of the A operand are staged per slab (256, or 128 when the tile holds
+// no more rows than that), always 256 rows of B.
+template <class E, int WMI, int WNJ, int AROWS>
+__device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const u32x4_t* __restrict__ wb,
+                                          uint16_t* __restrict__ y_tile, uint16_t* s_wide, int rows, int ncols,
+                                          int Kd, int N, int wm, int wn) {
   constexpr int TM = kWideM, TN = kWideN, BK = kWideK, LD = kWideLd, NT = kWideThreads;
-  extern __shared__ __attribute__((aligned(16))) uint16_t s_wide[];  // [2][TM + TN][LD]
-  __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
-  __shared__ int s_tmp[NT / kWave + 1];
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-
-  // (expert, m-tile, n-tile) of this workgroup, as in the 128 x 128 kernel with 256-row tiles
-  const int tile_n = blockIdx.x % ntile_n;
-  const int tile_m_global = blockIdx.x / ntile_n;
-  {
-    const int span = (num_experts + NT - 1) / NT;
-    const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
-    int sum = 0;
-    for (int e = lo; e < hi; ++e) sum += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
-    int total;
-    int run = block_exclusive_scan(sum, s_tmp, total);
-    for (int e = lo; e < hi; ++e) {
-      s_pref[e] = run;
-      run += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
-    }
-    if (tid == 0) s_pref[num_experts] = total;
-    __syncthreads();
-    if (tile_m_global >= total) return;
-  }
-  int e_lo = 0, e_hi = num_experts;
-  while (e_hi - e_lo > 1) {
-    int mid = (e_lo + e_hi) >> 1;
-    if (s_pref[mid] <= tile_m_global) e_lo = mid; else e_hi = mid;
-  }
-  const int e = e_lo;
-  const int count = offsets[e + 1] - offsets[e];
-  const int m0 = (tile_m_global - s_pref[e]) * TM;
-  const size_t row0 = (size_t)(max_recv > 0 ? e * max_recv : offsets[e]) + m0;
-  const int rows = min(TM, count - m0);
-  const int n0 = tile_n * TN;
-  const int ncols = min(TN, N - n0);
+  const int tid = threadIdx.x, lane = tid & (kWave - 1);
   const int kvec = Kd / 8;
-  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * kvec;
-  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * kvec;
-
-  // A slab is 256 rows x 8 vectors for each operand: eight vectors of each per thread.  Rows past
-  // the segment and columns past N read the last valid row instead of zeros: they only feed
-  // accumulators that are never stored, and the loads stay unconditional.
-  constexpr int VPR = BK / 8, NA = TM * VPR / NT, NB = TN * VPR / NT;
+  // A slab is AROWS (A) + 256 (B) rows x 8 vectors.  Rows past the segment and columns past N read
+  // the last valid row instead of zeros: they only feed accumulators that are never stored, and
+  // the loads stay unconditional.
+  constexpr int VPR = BK / 8, NA = AROWS * VPR / NT, NB = TN * VPR / NT;
   int offa[NA], offb[NB];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
@@ -1184,59 +1151,63 @@ __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const ui
         *reinterpret_cast<u32x4_t*>(&s_b_[i * (NT / VPR) * LD]) = rb[i];                                       \
   }
 
-  f32x16_t acc[4][4];
+  f32x16_t acc[WMI][WNJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < WMI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < WNJ; ++j)
 #pragma unroll
       for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
-  const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
   const int fr_a = (wm + (lane & 31)) * LD + (lane >> 5) * 8;
   const int fr_b = (TM + wn + (lane & 31)) * LD + (lane >> 5) * 8;
-  u32x4_t f0a[4], f0b[4], f1a[4], f1b[4];
+  u32x4_t f0a[WMI], f0b[WNJ], f1a[WMI], f1b[WNJ];
 #define WIDE_FRAGS(FA, FB, BUF, KK)                                                                            \
   {                                                                                                            \
     const uint16_t* base_ = s_wide + (BUF) * (TM + TN) * LD + (KK);                                            \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                              \
+    _Pragma("unroll") for (int i = 0; i < WMI; ++i)                                                            \
         FA[i] = *reinterpret_cast<const u32x4_t*>(&base_[fr_a + i * 32 * LD]);                                 \
-    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                              \
+    _Pragma("unroll") for (int j = 0; j < WNJ; ++j)                                                            \
         FB[j] = *reinterpret_cast<const u32x4_t*>(&base_[fr_b + j * 32 * LD]);                                 \
   }
 #define WIDE_MMA(FA, FB)                                                                                       \
   {                                                                                                            \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                              \
-    _Pragma("unroll") for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16_v<E>(FA[i], FB[j], acc[i][j]);     \
+    _Pragma("unroll") for (int i = 0; i < WMI; ++i)                                                            \
+    _Pragma("unroll") for (int j = 0; j < WNJ; ++j) acc[i][j] = mfma_32x32x16_v<E>(FA[i], FB[j], acc[i][j]);   \
   }
-  // instruction classes of the scheduling groups: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read, 0x200 LDS write
-#define WIDE_MIX_READS() /* 8 x (LDS read, MFMA), then the other 8 MFMAs */                                     \
+  // Instruction classes of the scheduling groups: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read,
+  // 0x200 LDS write.  Per step a wave issues MM MFMAs and RD fragment reads, per slab ST stores to
+  // LDS and ST global loads.
+  constexpr int RD = WMI + WNJ, MM = WMI * WNJ, ST = NA + NB;
+  constexpr int GW = wide_gcd(MM, ST), GF = wide_gcd(MM - RD, ST - RD);
+  static_assert(MM >= RD && ST >= RD, "interleave patterns assume at least one MFMA and one load per read");
+#define WIDE_MIX_READS() /* RD x (LDS read, MFMA), then the other MFMAs */                                      \
   {                                                                                                            \
-    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
+    _Pragma("unroll") for (int s_ = 0; s_ < RD; ++s_) {                                                        \
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                       \
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       \
     }                                                                                                          \
-    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);                                                         \
+    __builtin_amdgcn_sched_group_barrier(0x008, MM - RD, 0);                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                                         \
   }
-#define WIDE_MIX_WRITES() /* the 8 LDS reads, then 8 x (2 MFMA, 2 LDS writes) */                                \
+#define WIDE_MIX_WRITES() /* the LDS reads, then MFMAs and LDS writes in even shares */                         \
   {                                                                                                            \
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);                                                         \
-    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                                                       \
-      __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);                                                       \
+    __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);                                                        \
+    _Pragma("unroll") for (int s_ = 0; s_ < GW; ++s_) {                                                        \
+      __builtin_amdgcn_sched_group_barrier(0x008, MM / GW, 0);                                                 \
+      __builtin_amdgcn_sched_group_barrier(0x200, ST / GW, 0);                                                 \
     }                                                                                                          \
     __builtin_amdgcn_sched_barrier(0);                                                                         \
   }
-#define WIDE_MIX_FETCH() /* 8 x (LDS read, MFMA, global load), then 8 x (MFMA, global load) */                  \
+#define WIDE_MIX_FETCH() /* RD x (LDS read, MFMA, global load), then the rest in even shares */                 \
   {                                                                                                            \
-    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
+    _Pragma("unroll") for (int s_ = 0; s_ < RD; ++s_) {                                                        \
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                       \
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       \
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                       \
     }                                                                                                          \
-    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                         \
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       \
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                       \
+    _Pragma("unroll") for (int s_ = 0; s_ < GF; ++s_) {                                                        \
+      __builtin_amdgcn_sched_group_barrier(0x008, (MM - RD) / GF, 0);                                          \
+      __builtin_amdgcn_sched_group_barrier(0x020, (ST - RD) / GF, 0);                                          \
     }                                                                                                          \
     __builtin_amdgcn_sched_barrier(0);                                                                         \
   }
@@ -1276,16 +1247,70 @@ __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const ui
 #undef WIDE_MIX_FETCH
 
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < WMI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < WNJ; ++j)
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
         const int r = wm + i * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
         const int c = wn + j * 32 + (lane & 31);
-        if (r < rows && c < ncols)
-          y[(row0 + r) * (size_t)N + n0 + c] = (uint16_t)(E::pack(acc[i][j][q], 0.f) & 0xffffu);
+        if (r < rows && c < ncols) y_tile[r * (size_t)N + c] = (uint16_t)(E::pack(acc[i][j][q], 0.f) & 0xffffu);
       }
+}
+
+template <class E>
+__global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const uint4* __restrict__ x,
+                                                                         const uint4* __restrict__ w,
+                                                                         const int32_t* __restrict__ offsets,
+                                                                         uint16_t* __restrict__ y, int num_experts,
+                                                                         int Kd, int N, int max_recv, int ntile_n) {
+  constexpr int TM = kWideM, TN = kWideN, NT = kWideThreads;
+  extern __shared__ __attribute__((aligned(16))) uint16_t s_wide[];  // [2][TM + TN][LD]
+  __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
+  __shared__ int s_tmp[NT / kWave + 1];
+  const int tid = threadIdx.x, wave = tid / kWave;
+
+  // (expert, m-tile, n-tile) of this workgroup, as in the 128 x 128 kernel with 256-row tiles
+  const int tile_n = blockIdx.x % ntile_n;
+  const int tile_m_global = blockIdx.x / ntile_n;
+  {
+    const int span = (num_experts + NT - 1) / NT;
+    const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    int total;
+    int run = block_exclusive_scan(sum, s_tmp, total);
+    for (int e = lo; e < hi; ++e) {
+      s_pref[e] = run;
+      run += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    }
+    if (tid == 0) s_pref[num_experts] = total;
+    __syncthreads();
+    if (tile_m_global >= total) return;
+  }
+  int e_lo = 0, e_hi = num_experts;
+  while (e_hi - e_lo > 1) {
+    int mid = (e_lo + e_hi) >> 1;
+    if (s_pref[mid] <= tile_m_global) e_lo = mid; else e_hi = mid;
+  }
+  const int e = e_lo;
+  const int count = offsets[e + 1] - offsets[e];
+  const int m0 = (tile_m_global - s_pref[e]) * TM;
+  const size_t row0 = (size_t)(max_recv > 0 ? e * max_recv : offsets[e]) + m0;
+  const int rows = min(TM, count - m0);
+  const int n0 = tile_n * TN;
+  const int ncols = min(TN, N - n0);
+  const int kvec = Kd / 8;
+  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * kvec;
+  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * kvec;
+  uint16_t* y_tile = y + row0 * (size_t)N + n0;
+  // A segment's last tile is often less than half full (23 % of the MFMAs of a 512-rows-per-expert
+  // ragged input would be spent on rows that do not exist): up to 128 rows the four waves stand
+  // side by side on 128 x 64 each, and only 128 rows of A are staged.
+  if (rows > 128)
+    wide_tile<E, 4, 4, 256>(xa, wb, y_tile, s_wide, rows, ncols, Kd, N, (wave >> 1) * 128, (wave & 1) * 128);
+  else
+    wide_tile<E, 4, 2, 128>(xa, wb, y_tile, s_wide, rows, ncols, Kd, N, 0, wave * 64);
 }
 
 // ---------------------------------------------------------------------------------------
