@@ -237,7 +237,8 @@ def main():
     out = dict(
         metric=METRIC, value=round(value, 1), unit="GB/s", n_gpus=1, steps=timed_steps, warmup=args.warmup,
         ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
-        dtype="fp8-e4m3 dispatch, bf16 combine" if fp8 else str(cfg.in_dtype).replace("torch.", ""),
+        dtype="fp8-e4m3 dispatch, bf16 combine" if fp8 else {"bfloat16": "bf16", "float16": "f16"}[
+            str(cfg.in_dtype).replace("torch.", "")],
         data="synthetic",
         config=dict(workload=args.workload, tokens=T, experts=E, top_k=K, hidden=H, emulated_ranks=W,
                     routed_rows=T * K, combine=args.combine, launch="hipGraph replay, two steps per graph" if use_graph else "eager",
@@ -295,7 +296,8 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
 
     cfg = wl.cfg
     E, H, N = cfg.num_experts, cfg.hidden_dim, args.expert_gemm
-    ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind)
+    fp8 = wl.fp8_dispatch and not args.bf16_dispatch  # fp8 rows are dequantised inside the kernel
+    ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fp8_dispatch=fp8)
     gen = torch.Generator(device="cpu").manual_seed(1234)
     weights = (torch.randn(E, N, H, generator=gen) / H ** 0.5).to(cfg.in_dtype).to(dev)
     main = torch.cuda.Stream()
@@ -323,7 +325,8 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
                n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 5), higher_is_better=True,
                scaling="weak", vs_baseline=None, dtype="bf16" if cfg.in_dtype == torch.bfloat16 else "f16",
                data="synthetic",
-               config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N, kernel=kernel),
+               config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N, kernel=kernel,
+                           rows_dtype="fp8 e4m3fn + f32 scale per 128 columns" if fp8 else "16-bit"),
                kernels_us=summarise(per),
                roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
                              frac=round(tflops / MFMA_PEAK_TFLOPS, 4), traffic=None))
@@ -332,11 +335,16 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
 
         off = d.offsets.cpu()
         dx, wc, yg = d.disp_x.cpu(), weights.cpu(), y.cpu()
+        dsc = d.disp_scale.cpu() if fp8 else None
         t0, done, rows_done, worst = time.perf_counter(), 0, 0, 0.0
         for e in range(E):
             lo, hi = int(off[e]), int(off[e + 1])
             if hi > lo:
-                ref = O.expert_gemm(dx[lo:hi], torch.tensor([0, hi - lo], dtype=torch.int32), wc[e:e + 1], cfg.in_dtype)
+                seg = torch.tensor([0, hi - lo], dtype=torch.int32)
+                if fp8:
+                    ref = O.expert_gemm_fp8(dx[lo:hi], dsc[lo:hi], seg, wc[e:e + 1], cfg.in_dtype)
+                else:
+                    ref = O.expert_gemm(dx[lo:hi], seg, wc[e:e + 1], cfg.in_dtype)
                 want, got = ref.float(), yg[lo:hi].float()
                 # summation order differs from the CPU's: 1 % of the value + 1 % of the segment's rms
                 tol = 1e-2 * want.abs() + 1e-2 * want.pow(2).mean().sqrt()

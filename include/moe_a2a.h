@@ -193,6 +193,18 @@ int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offse
                         int N, int max_recv, int elem_type, moe_a2a_stream_t stream);
 
 /*
+ * The same product on rows that moe_a2a_dispatch_fp8 wrote: x_q[rows, Kd] e4m3fn bytes with
+ * x_scale[rows, Kd/128] f32.  A row element enters the product as elem(f32(q) * scale), i.e.
+ * dequantised and rounded once to the 16-bit type of the weights, inside the kernel (the rows
+ * are read as fp8: half the operand traffic, no dequantised copy in memory).  weights[E, N, Kd]
+ * and y[rows, N] are 16-bit elements of elem_type; Kd % 128 == 0, N % 8 == 0.  Always the
+ * 256 x 256 kernel.  No counterpart in the reference (it has no fp8 path).
+ */
+int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* weights, const int32_t* offsets,
+                            void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
+                            moe_a2a_stream_t stream);
+
+/*
  * Launch timer (opt-in, process-wide, single caller thread).  Between begin and end every
  * kernel the library launches carries a pair of HIP events bound to that dispatch, so the
  * reported time is the kernel's own begin-to-end duration on the GPU.

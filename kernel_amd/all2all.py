@@ -233,27 +233,35 @@ class HipAllToAll:
         """Real expert compute in place of the stub: ``y[rows of e] = disp_x[rows of e] @ weights[e].T``
         for every expert, on the matrix cores (f32 accumulation, one rounding to ``out_dtype``).
 
-        ``weights[E, N, H]`` of ``in_dtype``; returns ``y[rows, N]`` with the row layout of the
+        ``weights[E, N, H]`` of ``out_dtype``; returns ``y[rows, N]`` with the row layout of the
         dispatched buffer (rows that hold no entry are not written).  ``N == H`` feeds ``combine``.
+        16-bit dispatched rows must have the weights' type; fp8 dispatched rows (``d.disp_scale``
+        set) are dequantised inside the kernel, each element rounded once to the weights' type.
         """
         cfg = self.cfg
-        if d.disp_scale is not None:
-            raise ValueError("expert_gemm takes 16-bit dispatched rows")
         _require_gpu(weights, "weights")
         rows, H = d.disp_x.shape
         E = cfg.num_experts
-        if weights.dim() != 3 or weights.shape[0] != E or weights.shape[2] != H or weights.dtype != d.disp_x.dtype:
-            raise ValueError("weights must be in_dtype[E, N, H]")
-        if cfg.out_dtype != d.disp_x.dtype:
-            raise ValueError("expert_gemm keeps the element type of the dispatched rows")
+        if weights.dim() != 3 or weights.shape[0] != E or weights.shape[2] != H or weights.dtype != cfg.out_dtype \
+                or not weights.is_contiguous():
+            raise ValueError("weights must be out_dtype[E, N, H], contiguous")
+        fp8 = d.disp_scale is not None
+        if not fp8 and cfg.out_dtype != d.disp_x.dtype:
+            raise ValueError("expert_gemm keeps the element type of 16-bit dispatched rows")
         N = weights.shape[1]
         if out is None:
             out = torch.empty(rows, N, dtype=cfg.out_dtype, device=weights.device)
         elif tuple(out.shape) != (rows, N) or out.dtype != cfg.out_dtype or not out.is_contiguous():
             raise ValueError("out must be out_dtype[rows, N], contiguous")
-        _lib.check(self.lib.moe_a2a_expert_gemm(_ptr(d.disp_x), _ptr(weights), _ptr(d.offsets), _ptr(out),
-                                                d.num_rows, E, H, N, d.max_recv, _elem(cfg.out_dtype), _stream()),
-                   "moe_a2a_expert_gemm")
+        if fp8:
+            _lib.check(self.lib.moe_a2a_expert_gemm_fp8(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(weights),
+                                                        _ptr(d.offsets), _ptr(out), d.num_rows, E, H, N, d.max_recv,
+                                                        _elem(cfg.out_dtype), _stream()),
+                       "moe_a2a_expert_gemm_fp8")
+        else:
+            _lib.check(self.lib.moe_a2a_expert_gemm(_ptr(d.disp_x), _ptr(weights), _ptr(d.offsets), _ptr(out),
+                                                    d.num_rows, E, H, N, d.max_recv, _elem(cfg.out_dtype), _stream()),
+                       "moe_a2a_expert_gemm")
         return out
 
     # ---- combine ---------------------------------------------------------------------

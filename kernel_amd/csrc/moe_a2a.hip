@@ -1107,25 +1107,48 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16_v<F16>(const u32x4_t& a, const
 
 constexpr int wide_gcd(int a, int b) { return b == 0 ? a : wide_gcd(b, a % b); }
 
+// 16 fp8 (e4m3fn) values and their block scale -> two vectors of 8 values of E: E(f32(q) * scale)
+template <class E>
+__device__ __forceinline__ void wide_decode_fp8(const u32x4_t& q, float scale, u32x4_t& lo, u32x4_t& hi) {
+  uint32_t o[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float f[4];
+    fp8x4_to_f32(q[j], f);
+    o[2 * j] = E::pack(f[0] * scale, f[1] * scale);
+    o[2 * j + 1] = E::pack(f[2] * scale, f[3] * scale);
+  }
+  lo = u32x4_t{o[0], o[1], o[2], o[3]};
+  hi = u32x4_t{o[4], o[5], o[6], o[7]};
+}
+
 // Main loop and epilogue of one wide tile.  Each wave owns WMI x WNJ accumulator blocks of 32 x 32
 // at (wm, wn); AROWS rows of the A operand are staged per slab (256, or 128 when the tile holds
 // no more rows than that), always 256 rows of B.
-template <class E, int WMI, int WNJ, int AROWS>
-__device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const u32x4_t* __restrict__ wb,
-                                          uint16_t* __restrict__ y_tile, uint16_t* s_wide, int rows, int ncols,
-                                          int Kd, int N, int wm, int wn) {
+template <class E, int WMI, int WNJ, int AROWS, bool AFP8>
+__device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const float* __restrict__ xs,
+                                          const u32x4_t* __restrict__ wb, uint16_t* __restrict__ y_tile,
+                                          uint16_t* s_wide, int rows, int ncols, int Kd, int N, int wm, int wn) {
   constexpr int TM = kWideM, TN = kWideN, BK = kWideK, LD = kWideLd, NT = kWideThreads;
   const int tid = threadIdx.x, lane = tid & (kWave - 1);
   const int kvec = Kd / 8;
-  // A slab is AROWS (A) + 256 (B) rows x 8 vectors.  Rows past the segment and columns past N read
-  // the last valid row instead of zeros: they only feed accumulators that are never stored, and
-  // the loads stay unconditional.
-  constexpr int VPR = BK / 8, NA = AROWS * VPR / NT, NB = TN * VPR / NT;
-  int offa[NA], offb[NB];
+  // A slab is AROWS (A) + 256 (B) rows of 64 elements.  Rows past the segment and columns past N
+  // read the last valid row instead of zeros: they only feed accumulators that are never stored,
+  // and the loads stay unconditional.  16-bit A: 8 vectors of 8 elements per row.  fp8 A (AFP8): 4
+  // vectors of 16 elements per row plus the row's f32 scale of that 128-column block; a vector is
+  // turned into two 16-bit vectors, E(f32(q) * scale), on its way into LDS, so the LDS image, the
+  // number of LDS stores and the number of global loads per thread are those of the 16-bit case.
+  constexpr int VPR = BK / 8, NB = TN * VPR / NT;
+  constexpr int AVPR = AFP8 ? BK / 16 : VPR;      // global A vectors per row and slab
+  constexpr int NA = AROWS * AVPR / NT;            // ... per thread
+  constexpr int NS = AFP8 ? NA : 0;                // scales per thread
+  int offa[NA], offs[NS > 0 ? NS : 1], offb[NB];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
     const int v = tid + i * NT;
-    offa[i] = min(v / VPR, rows - 1) * kvec + v % VPR;
+    const int r = min(v / AVPR, rows - 1);
+    offa[i] = r * (AFP8 ? Kd / 16 : kvec) + v % AVPR;
+    if (AFP8) offs[i] = r * (Kd / 128);
   }
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
@@ -1134,19 +1157,30 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
   }
   // native vectors, not uint4: the struct type keeps the staging arrays in scratch memory
   u32x4_t ra[NA], rb[NB];
+  float rs[NS > 0 ? NS : 1];
   const int st_off = (tid / VPR) * LD + (tid % VPR) * 8;
-#define WIDE_FETCH(K0)                                                           \
-  {                                                                              \
-    const int kv_ = (K0) >> 3;                                                   \
-    _Pragma("unroll") for (int i = 0; i < NA; ++i) ra[i] = xa[offa[i] + kv_];    \
-    _Pragma("unroll") for (int i = 0; i < NB; ++i) rb[i] = wb[offb[i] + kv_];    \
+  const int st_off_a = AFP8 ? (tid / AVPR) * LD + (tid % AVPR) * 16 : st_off;
+#define WIDE_FETCH(K0)                                                                           \
+  {                                                                                              \
+    const int kv_ = (K0) >> (AFP8 ? 4 : 3);                                                      \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i) ra[i] = xa[offa[i] + kv_];                    \
+    if (AFP8) { _Pragma("unroll") for (int i = 0; i < NS; ++i) rs[i] = xs[offs[i] + ((K0) >> 7)]; } \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) rb[i] = wb[offb[i] + ((K0) >> 3)];            \
   }
 #define WIDE_STASH(BUF)                                                                                        \
   {                                                                                                            \
-    uint16_t* s_a_ = s_wide + (BUF) * (TM + TN) * LD + st_off;                                                 \
-    uint16_t* s_b_ = s_a_ + TM * LD;                                                                           \
-    _Pragma("unroll") for (int i = 0; i < NA; ++i)                                                             \
-        *reinterpret_cast<u32x4_t*>(&s_a_[i * (NT / VPR) * LD]) = ra[i];                                       \
+    uint16_t* s_a_ = s_wide + (BUF) * (TM + TN) * LD + st_off_a;                                               \
+    uint16_t* s_b_ = s_wide + (BUF) * (TM + TN) * LD + TM * LD + st_off;                                       \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i) {                                                           \
+      if (AFP8) {                                                                                              \
+        u32x4_t lo_, hi_;                                                                                      \
+        wide_decode_fp8<E>(ra[i], rs[i], lo_, hi_);                                                            \
+        *reinterpret_cast<u32x4_t*>(&s_a_[i * (NT / AVPR) * LD]) = lo_;                                        \
+        *reinterpret_cast<u32x4_t*>(&s_a_[i * (NT / AVPR) * LD + 8]) = hi_;                                    \
+      } else {                                                                                                 \
+        *reinterpret_cast<u32x4_t*>(&s_a_[i * (NT / AVPR) * LD]) = ra[i];                                      \
+      }                                                                                                        \
+    }                                                                                                          \
     _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                             \
         *reinterpret_cast<u32x4_t*>(&s_b_[i * (NT / VPR) * LD]) = rb[i];                                       \
   }
@@ -1177,7 +1211,7 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
   // Instruction classes of the scheduling groups: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read,
   // 0x200 LDS write.  Per step a wave issues MM MFMAs and RD fragment reads, per slab ST stores to
   // LDS and ST global loads.
-  constexpr int RD = WMI + WNJ, MM = WMI * WNJ, ST = NA + NB;
+  constexpr int RD = WMI + WNJ, MM = WMI * WNJ, ST = (AFP8 ? 2 * NA : NA) + NB;  // LDS stores == global loads
   constexpr int GW = wide_gcd(MM, ST), GF = wide_gcd(MM - RD, ST - RD);
   static_assert(MM >= RD && ST >= RD, "interleave patterns assume at least one MFMA and one load per read");
 #define WIDE_MIX_READS() /* RD x (LDS read, MFMA), then the other MFMAs */                                      \
@@ -1258,8 +1292,9 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
       }
 }
 
-template <class E>
+template <class E, bool AFP8>
 __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const uint4* __restrict__ x,
+                                                                         const float* __restrict__ x_scale,
                                                                          const uint4* __restrict__ w,
                                                                          const int32_t* __restrict__ offsets,
                                                                          uint16_t* __restrict__ y, int num_experts,
@@ -1301,16 +1336,18 @@ __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const ui
   const int n0 = tile_n * TN;
   const int ncols = min(TN, N - n0);
   const int kvec = Kd / 8;
-  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * kvec;
+  // fp8 rows are Kd bytes (Kd / 16 vectors) with Kd / 128 scales each
+  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * (AFP8 ? Kd / 16 : kvec);
+  const float* xs = AFP8 ? x_scale + row0 * (Kd / 128) : nullptr;
   const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * kvec;
   uint16_t* y_tile = y + row0 * (size_t)N + n0;
   // A segment's last tile is often less than half full (23 % of the MFMAs of a 512-rows-per-expert
   // ragged input would be spent on rows that do not exist): up to 128 rows the four waves stand
   // side by side on 128 x 64 each, and only 128 rows of A are staged.
   if (rows > 128)
-    wide_tile<E, 4, 4, 256>(xa, wb, y_tile, s_wide, rows, ncols, Kd, N, (wave >> 1) * 128, (wave & 1) * 128);
+    wide_tile<E, 4, 4, 256, AFP8>(xa, xs, wb, y_tile, s_wide, rows, ncols, Kd, N, (wave >> 1) * 128, (wave & 1) * 128);
   else
-    wide_tile<E, 4, 2, 128>(xa, wb, y_tile, s_wide, rows, ncols, Kd, N, 0, wave * 64);
+    wide_tile<E, 4, 2, 128, AFP8>(xa, xs, wb, y_tile, s_wide, rows, ncols, Kd, N, 0, wave * 64);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1741,6 +1778,37 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   return moe_a2a_combine(expert_y, weights, slot_of_entry, combine_mode, out_type, out, T, K, H, stream);
 }
 
+// Launch of the 256 x 256 kernel; x_scale != nullptr selects fp8 rows of x.
+static int launch_gemm_wide(const void* x, const float* x_scale, const void* weights, const int32_t* offsets, void* y,
+                            int R, int E, int Kd, int N, int max_recv, int elem_type, hipStream_t stream) {
+  const int ntile_n = ceil_div(N, kWideN);
+  const long long mtiles = (long long)R / kWideM + E;  // every expert may end with a partly filled tile
+  if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
+  dim3 grid((unsigned)(mtiles * ntile_n)), block(kWideThreads);
+  static bool lds_raised = false;  // the kernels need more dynamic LDS than the 64 KB default
+  if (!lds_raised) {
+    const void* kernels[4] = {(const void*)expert_gemm_wide_kernel<Bf16, false>,
+                              (const void*)expert_gemm_wide_kernel<F16, false>,
+                              (const void*)expert_gemm_wide_kernel<Bf16, true>,
+                              (const void*)expert_gemm_wide_kernel<F16, true>};
+    for (const void* k : kernels) {
+      hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
+      if (e != hipSuccess) return (int)e;
+    }
+    lds_raised = true;
+  }
+#define CALL_WIDE(ET, FP8)                                                                                     \
+  return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<ET, FP8>, grid, block, kWideLdsBytes, stream,    \
+                (const uint4*)x, x_scale, (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n)
+  if (x_scale) {
+    if (elem_type == MOE_A2A_BF16) CALL_WIDE(Bf16, true);
+    CALL_WIDE(F16, true);
+  }
+  if (elem_type == MOE_A2A_BF16) CALL_WIDE(Bf16, false);
+  CALL_WIDE(F16, false);
+#undef CALL_WIDE
+}
+
 int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offsets, void* y, int R, int E, int Kd,
                         int N, int max_recv, int elem_type, moe_a2a_stream_t stream_) {
   if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
@@ -1755,26 +1823,7 @@ int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offse
   // of its tiles would be half empty.  MOE_A2A_GEMM_TILE=128|256 in the environment overrides.
   bool wide = (long long)R >= 256ll * E && N >= kWideN;
   if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) wide = atoi(forced) == 256;
-  if (wide) {
-    const int ntile_n = ceil_div(N, kWideN);
-    const long long mtiles = (long long)R / kWideM + E;  // every expert may end with a partly filled tile
-    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-    dim3 grid((unsigned)(mtiles * ntile_n)), block(kWideThreads);
-    static bool lds_raised = false;  // the kernels need more dynamic LDS than the 64 KB default
-    if (!lds_raised) {
-      hipError_t e1 = hipFuncSetAttribute((const void*)expert_gemm_wide_kernel<Bf16>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
-      hipError_t e2 = hipFuncSetAttribute((const void*)expert_gemm_wide_kernel<F16>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
-      if (e1 != hipSuccess || e2 != hipSuccess) return (int)(e1 != hipSuccess ? e1 : e2);
-      lds_raised = true;
-    }
-    if (elem_type == MOE_A2A_BF16)
-      return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<Bf16>, grid, block, kWideLdsBytes, stream,
-                    (const uint4*)x, (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-    return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<F16>, grid, block, kWideLdsBytes, stream,
-                  (const uint4*)x, (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-  }
+  if (wide) return launch_gemm_wide(x, nullptr, weights, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
   const int ntile_n = ceil_div(N, kGemmN);
   // worst case of m-tiles: every expert ends with a partly filled tile
   const long long mtiles = (long long)R / kGemmM + E;
@@ -1785,6 +1834,19 @@ int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offse
                   (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
   return launch(KID_EXPERT_GEMM, expert_gemm_kernel<F16>, grid, block, 0, stream, (const uint4*)x,
                 (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+}
+
+int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* weights, const int32_t* offsets,
+                            void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
+                            moe_a2a_stream_t stream_) {
+  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
+  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 || N < 8 ||
+      N % 8 != 0 || max_recv < 0)
+    return MOE_A2A_E_SHAPE;
+  if (R == 0) return 0;
+  if (!x_q || !x_scale || !weights || !offsets || !y) return MOE_A2A_E_NULL;
+  if (!aligned16(x_q) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
+  return launch_gemm_wide(x_q, x_scale, weights, offsets, y, R, E, Kd, N, max_recv, elem_type, (hipStream_t)stream_);
 }
 
 int moe_a2a_timer_begin(int capacity) {

@@ -144,6 +144,14 @@ def expert_gemm(disp_x: torch.Tensor, offsets: torch.Tensor, weights: torch.Tens
     return y
 
 
+def expert_gemm_fp8(q_bits: torch.Tensor, scale: torch.Tensor, offsets: torch.Tensor, weights: torch.Tensor,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """The same layer on fp8 dispatched rows: each element is dequantised, ``f32(q) * scale``, and
+    rounded once to the weights' 16-bit type before it enters the product (what the HIP kernel
+    stages into LDS).  No counterpart in the reference."""
+    return expert_gemm(dequantize_fp8(q_bits, scale).to(weights.dtype), offsets, weights, out_dtype)
+
+
 def combine_strict(expert_y: torch.Tensor, weights: torch.Tensor, slot_of_entry: torch.Tensor,
                    out_dtype: torch.dtype) -> torch.Tensor:
     """Reference-order weighted sum with a rounding to ``out_dtype`` after every add."""

@@ -106,6 +106,29 @@ def test_row_functions_reject_bad_arguments(lib):
     assert lib.moe_a2a_route_dispatch(A, A, None, 0, big, 8, 8, 2, 64, 0, A, A, A, A, A, None, A, None) == E_SHAPE
 
 
+def test_expert_gemm_rejects_bad_arguments(lib):
+    def gemm(x=A, w=A, off=A, y=A, R=64, E=8, Kd=128, N=64, max_recv=0, elem=_lib.BF16):
+        return lib.moe_a2a_expert_gemm(x, w, off, y, R, E, Kd, N, max_recv, elem, None)
+
+    def gemm8(x=A, sc=A, w=A, off=A, y=A, R=64, E=8, Kd=128, N=64, max_recv=0, elem=_lib.BF16):
+        return lib.moe_a2a_expert_gemm_fp8(x, sc, w, off, y, R, E, Kd, N, max_recv, elem, None)
+
+    for f in (gemm, gemm8):
+        assert f(elem=5) == E_DTYPE
+        assert f(E=0) == E_SHAPE
+        assert f(E=1025) == E_SHAPE
+        assert f(N=12) == E_SHAPE
+        assert f(max_recv=-1) == E_SHAPE
+        assert f(R=-1) == E_SHAPE
+        assert f(R=0) == 0  # nothing to do, nothing launched
+        assert f(w=None) == E_NULL
+        assert f(off=None) == E_NULL
+        assert f(y=A + 8) == E_ALIGN
+    assert gemm(Kd=72) == E_SHAPE    # hidden size in slabs of 64
+    assert gemm8(Kd=192) == E_SHAPE  # fp8 rows carry one scale per 128 columns
+    assert gemm8(sc=None) == E_NULL
+
+
 def test_timer_needs_begin_first(lib):
     ids = (ctypes.c_int * 4)()
     us = (ctypes.c_float * 4)()

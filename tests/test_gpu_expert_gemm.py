@@ -95,6 +95,46 @@ def test_both_tile_sizes_give_the_same_bits(gpu_device, monkeypatch, E, K, T, H,
     close(outs["256"], V.expert_gemm(o["disp_x"], o["offsets"], weights, dtype))
 
 
+@pytest.mark.parametrize("E,K,T,H,N,W,zipf", [
+    (8, 2, 40, 128, 64, 1, False),      # one scale block, tiles mostly empty
+    (8, 2, 1200, 256, 264, 2, False),   # full 256-row tiles and 128-row tails, ragged N
+    (16, 4, 300, 384, 136, 4, True),    # skewed: empty experts and long segments
+    (32, 4, 2048, 1024, 512, 8, False),
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
+def test_expert_gemm_on_fp8_rows(gpu_device, E, K, T, H, N, W, zipf, dtype, padded):
+    """fp8 dispatch -> expert GEMM.  The dispatched bytes and scales are bit-exact (checked here
+    again), and the product is compared with an f32 matmul of the dequantised rows, each element
+    rounded once to the weights' type as the kernel does."""
+    cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=3 * E + T, zipf=zipf)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, fp8_dispatch=True, padded=padded, max_recv=T if padded else None)
+    d = ata.dispatch(x, idx, rs)
+    y = ata.expert_gemm(d, weights.to(gpu_device))
+    torch.cuda.synchronize()
+    o = V.run_world(cfg, world, fp8=True)
+    rows = d.slot_of_entry.long() if padded else o["slot_of_entry"].long().to(gpu_device)
+    soe = o["slot_of_entry"].long()
+    assert torch.equal(d.disp_x[rows].cpu(), o["disp_x"][soe])
+    assert torch.equal(d.disp_scale[rows].cpu(), o["disp_scale"][soe])
+    want = V.expert_gemm_fp8(o["disp_x"], o["disp_scale"], o["offsets"], weights, dtype)
+    close(y[rows], want[soe])
+
+
+def test_fp8_gemm_feeds_combine(gpu_device):
+    """fp8 dispatch -> expert GEMM (H -> H) -> f32 combine against the same chain on the CPU."""
+    cfg, world, weights = make(32, 4, 1024, 256, 256, 8, torch.bfloat16, seed=5)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, 8, fp8_dispatch=True, combine_mode=C.COMBINE_F32)
+    d = ata.dispatch(x, idx, rs)
+    y = ata.combine(None, w, d, ata.expert_gemm(d, weights.to(gpu_device)))
+    o = V.run_world(cfg, world, fp8=True)
+    ey = V.expert_gemm_fp8(o["disp_x"], o["disp_scale"], o["offsets"], weights, torch.bfloat16)
+    want = V.combine_f32(ey, w.cpu(), o["slot_of_entry"], torch.bfloat16)
+    close(y, want)
+
+
 def test_dispatch_gemm_combine_end_to_end(gpu_device):
     """dispatch -> expert GEMM (H -> H) -> combine against the same chain on the CPU."""
     cfg, world, weights = make(32, 4, 512, 256, 256, 8, torch.bfloat16, seed=3)
