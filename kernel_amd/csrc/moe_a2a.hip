@@ -2,8 +2,10 @@
 //
 // The W destination ranks of the reference's all-to-all (all2all/reference.py:68-234) are
 // partitions of one compact expert-major buffer, so an "exchange" is only the choice of a
-// destination row.  Everything here is HBM-bound integer/byte work: no MFMA, 16-byte
-// vector loads and stores, LDS for counters and index tiles, ballot/popcount for ranks.
+// destination row.  The dispatch/combine path is HBM-bound integer/byte work: no MFMA, 16-byte
+// vector loads and stores, LDS for counters and index tiles, ballot/popcount for ranks.  The
+// expert layer that a real model runs between the two (the reference has a scalar stub there) is
+// the one matrix-core kernel family: a grouped GEMM over the dispatched segments.
 //
 // Kernels
 //   route_*            histogram, exclusive scan, stable permutation, meta rows
@@ -12,10 +14,14 @@
 //   dispatch_fp8       same copy with e4m3fn quantisation per 128 columns
 //   stub_*             expert stand-in, one factor per row
 //   combine / stub_combine   gather K rows per token, weighted sum
+//   expert_gemm        y[rows of e] = x[rows of e] * W_e^T, 128 x 128 tiles (short segments)
+//   expert_gemm_wide   the same on 256 x 256 tiles, software-pipelined; 16-bit or fp8 rows
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdlib.h>
+
+#include <atomic>
 
 #include "moe_a2a.h"
 
@@ -1105,6 +1111,7 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16_v<F16>(const u32x4_t& a, const
                                                 0, 0);
 }
 
+constexpr int kMaxDevices = 64;
 constexpr int wide_gcd(int a, int b) { return b == 0 ? a : wide_gcd(b, a % b); }
 
 // 16 fp8 (e4m3fn) values and their block scale -> two vectors of 8 values of E: E(f32(q) * scale)
@@ -1785,8 +1792,13 @@ static int launch_gemm_wide(const void* x, const float* x_scale, const void* wei
   const long long mtiles = (long long)R / kWideM + E;  // every expert may end with a partly filled tile
   if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
   dim3 grid((unsigned)(mtiles * ntile_n)), block(kWideThreads);
-  static bool lds_raised = false;  // the kernels need more dynamic LDS than the 64 KB default
-  if (!lds_raised) {
+  // the kernels need more dynamic LDS than the 64 KB default: raised once per device (the
+  // attribute belongs to the device's copy of the function); racing first calls only repeat it
+  static std::atomic<bool> lds_raised[kMaxDevices];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return MOE_A2A_E_STATE;
+  if (!lds_raised[dev].load(std::memory_order_acquire)) {
     const void* kernels[4] = {(const void*)expert_gemm_wide_kernel<Bf16, false>,
                               (const void*)expert_gemm_wide_kernel<F16, false>,
                               (const void*)expert_gemm_wide_kernel<Bf16, true>,
@@ -1795,7 +1807,7 @@ static int launch_gemm_wide(const void* x, const float* x_scale, const void* wei
       hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
       if (e != hipSuccess) return (int)e;
     }
-    lds_raised = true;
+    lds_raised[dev].store(true, std::memory_order_release);
   }
 #define CALL_WIDE(ET, FP8)                                                                                     \
   return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<ET, FP8>, grid, block, kWideLdsBytes, stream,    \
