@@ -186,8 +186,9 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
  * this is the grouped matrix product a real MoE layer runs there.
  *   x[rows, Kd], weights[E, N, Kd], y[rows, N]: 16-bit elements of elem_type, f32 accumulation,
  *   Kd % 64 == 0, N % 8 == 0, 16-byte aligned.
- * Two kernels with identical results: 128 x 128 output tiles, and 256 x 256 tiles when segments are
- * long (R >= 256 * E and N >= 256).  MOE_A2A_GEMM_TILE=128 or 256 in the environment forces one.
+ * Three kernels with identical results: 128 x 128 output tiles; 256 x 256 tiles when segments are
+ * long (R >= 256 * E and N >= 256); 32 x 128 tiles that stream the weights when segments are short
+ * (R <= 32 * E and Kd % 128 == 0).  MOE_A2A_GEMM_TILE=32, 128 or 256 in the environment forces one.
  */
 int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offsets, void* y, int R, int E, int Kd,
                         int N, int max_recv, int elem_type, moe_a2a_stream_t stream);

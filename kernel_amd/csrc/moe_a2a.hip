@@ -52,12 +52,13 @@ enum KernelId {
   KID_STUB_COMBINE,
   KID_EXPERT_GEMM,
   KID_EXPERT_GEMM_WIDE,
+  KID_EXPERT_GEMM_SKINNY,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
-    "expert_gemm_wide"};
+    "expert_gemm_wide", "expert_gemm_skinny"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -1111,6 +1112,146 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16_v<F16>(const u32x4_t& a, const
                                                 0, 0);
 }
 
+// Skinny variant for short segments (a decode step: a handful of rows per expert).  The work is
+// then streaming each expert's weights once: 32 x 128 output tiles (one row block, so 4x fewer
+// MFMAs are spent on rows that do not exist than with 128-row tiles), four waves side by side on
+// 32 x 32 each, K slabs of 128 (256 contiguous bytes of every weight row per slab: measured 6.09
+// TB/s of weights at 256 experts x 8 rows, 7168 -> 2048, against 5.95 with 256 x 64 slabs and 5.84
+// for the 128 x 128 kernel), and the global -> register prefetch runs TWO slabs ahead in two
+// register sets.  Accumulation order over K equals the other kernels': same bits.
+constexpr int kSkinnyM = 32, kSkinnyThreads = 256;
+#ifndef MOE_A2A_SKINNY_N
+#define MOE_A2A_SKINNY_N 128
+#define MOE_A2A_SKINNY_K 128
+#endif
+constexpr int kSkinnyN = MOE_A2A_SKINNY_N, kSkinnyK = MOE_A2A_SKINNY_K;
+
+template <class E>
+__global__ __launch_bounds__(kSkinnyThreads, 3) void expert_gemm_skinny_kernel(const uint4* __restrict__ x,
+                                                                            const uint4* __restrict__ w,
+                                                                            const int32_t* __restrict__ offsets,
+                                                                            uint16_t* __restrict__ y, int num_experts,
+                                                                            int Kd, int N, int max_recv, int ntile_n) {
+  constexpr int TM = kSkinnyM, TN = kSkinnyN, BK = kSkinnyK, LD = BK + 8, NT = kSkinnyThreads;  // Kd % BK == 0
+  constexpr int WJ = TN / 128;  // 32-column blocks per wave
+  __shared__ __attribute__((aligned(16))) uint16_t s_ab[(TM + TN) * LD];
+  uint16_t* s_a = s_ab;
+  uint16_t* s_b = s_ab + TM * LD;
+  __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
+  __shared__ int s_tmp[NT / kWave + 1];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+
+  const int tile_n = blockIdx.x % ntile_n;
+  const int tile_m_global = blockIdx.x / ntile_n;
+  {
+    const int span = (num_experts + NT - 1) / NT;
+    const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    int total;
+    int run = block_exclusive_scan(sum, s_tmp, total);
+    for (int e = lo; e < hi; ++e) {
+      s_pref[e] = run;
+      run += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    }
+    if (tid == 0) s_pref[num_experts] = total;
+    __syncthreads();
+    if (tile_m_global >= total) return;
+  }
+  int e_lo = 0, e_hi = num_experts;
+  while (e_hi - e_lo > 1) {
+    int mid = (e_lo + e_hi) >> 1;
+    if (s_pref[mid] <= tile_m_global) e_lo = mid; else e_hi = mid;
+  }
+  const int e = e_lo;
+  const int count = offsets[e + 1] - offsets[e];
+  const int m0 = (tile_m_global - s_pref[e]) * TM;
+  const size_t row0 = (size_t)(max_recv > 0 ? e * max_recv : offsets[e]) + m0;
+  const int rows = min(TM, count - m0);
+  const int n0 = tile_n * TN;
+  const int ncols = min(TN, N - n0);
+  const int kvec = Kd / 8;
+  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * kvec;
+  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * kvec;
+
+  // per slab: one vector of A (32 rows x 8) and eight of B (256 rows x 8) per thread; rows past
+  // the segment / columns past N read the last valid one (they feed accumulators never stored)
+  constexpr int VPR = BK / 8, NB = TN * VPR / NT;
+  constexpr int NA = TM * VPR / NT > 0 ? TM * VPR / NT : 1;
+  int offa[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int v = tid + i * NT;
+    offa[i] = min(v / VPR, rows - 1) * kvec + v % VPR;
+  }
+  int offb[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int v = tid + i * NT;
+    offb[i] = min(v / VPR, ncols - 1) * kvec + v % VPR;
+  }
+  const int st_off = (tid / VPR) * LD + (tid % VPR) * 8;
+  u32x4_t ra0[NA], rb0[NB], ra1[NA], rb1[NB];
+#define SKINNY_FETCH(RA, RB, K0)                                               \
+  {                                                                            \
+    const int kv_ = min((K0), Kd - BK) >> 3; /* past the end: the last slab again */ \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i) RA[i] = xa[offa[i] + kv_];  \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) RB[i] = wb[offb[i] + kv_];  \
+  }
+#define SKINNY_STASH(RA, RB)                                                                          \
+  {                                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i)                                                    \
+        *reinterpret_cast<u32x4_t*>(&s_a[st_off + i * (NT / VPR) * LD]) = RA[i];                      \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                    \
+        *reinterpret_cast<u32x4_t*>(&s_b[st_off + i * (NT / VPR) * LD]) = RB[i];                      \
+  }
+  f32x16_t acc[WJ];
+#pragma unroll
+  for (int j = 0; j < WJ; ++j)
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc[j][q] = 0.f;
+  const int wn = wave * 32 * WJ;
+  const int fr_a = (lane & 31) * LD + (lane >> 5) * 8;
+  const int fr_b = (wn + (lane & 31)) * LD + (lane >> 5) * 8;
+#define SKINNY_SLAB()                                                                                 \
+  {                                                                                                   \
+    _Pragma("unroll") for (int kk = 0; kk < BK; kk += 16) {                                           \
+      const u32x4_t fa = *reinterpret_cast<const u32x4_t*>(&s_a[fr_a + kk]);                          \
+      _Pragma("unroll") for (int j = 0; j < WJ; ++j) {                                                 \
+        const u32x4_t fb = *reinterpret_cast<const u32x4_t*>(&s_b[fr_b + j * 32 * LD + kk]);          \
+        acc[j] = mfma_32x32x16_v<E>(fa, fb, acc[j]);                                                  \
+      }                                                                                               \
+    }                                                                                                 \
+  }
+  SKINNY_FETCH(ra0, rb0, 0);
+  SKINNY_FETCH(ra1, rb1, BK);
+  for (int k0 = 0; k0 < Kd; k0 += 2 * BK) {
+    SKINNY_STASH(ra0, rb0);
+    __syncthreads();
+    SKINNY_FETCH(ra0, rb0, k0 + 2 * BK);
+    SKINNY_SLAB();
+    __syncthreads();
+    if (k0 + BK >= Kd) break;
+    SKINNY_STASH(ra1, rb1);
+    __syncthreads();
+    SKINNY_FETCH(ra1, rb1, k0 + 3 * BK);
+    SKINNY_SLAB();
+    __syncthreads();
+  }
+#undef SKINNY_FETCH
+#undef SKINNY_STASH
+#undef SKINNY_SLAB
+#pragma unroll
+  for (int j = 0; j < WJ; ++j)
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int r = (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
+      const int c = wn + j * 32 + (lane & 31);
+      if (r < rows && c < ncols)
+        y[(row0 + r) * (size_t)N + n0 + c] = (uint16_t)(E::pack(acc[j][q], 0.f) & 0xffffu);
+    }
+}
+
 constexpr int kMaxDevices = 64;
 constexpr int wide_gcd(int a, int b) { return b == 0 ? a : wide_gcd(b, a % b); }
 
@@ -1832,10 +1973,27 @@ int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offse
   if (!aligned16(x) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
   hipStream_t stream = (hipStream_t)stream_;
   // Long segments take the 256 x 256 kernel: with fewer than 256 rows per expert on average most
-  // of its tiles would be half empty.  MOE_A2A_GEMM_TILE=128|256 in the environment overrides.
+  // of its tiles would be half empty.  MOE_A2A_GEMM_TILE=32|128|256 in the environment overrides.
+  // Short segments (a decode step) take the 32 x 256 kernel, which streams the weights.
   bool wide = (long long)R >= 256ll * E && N >= kWideN;
-  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) wide = atoi(forced) == 256;
+  bool skinny = (long long)R <= 32ll * E;
+  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) {
+    wide = atoi(forced) == 256;
+    skinny = atoi(forced) == 32;
+  }
+  if (Kd % kSkinnyK != 0) skinny = false;  // its K slabs are 128 wide; the 128 x 128 kernel takes the rest
   if (wide) return launch_gemm_wide(x, nullptr, weights, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
+  if (skinny) {
+    const int ntile_n = ceil_div(N, kSkinnyN);
+    const long long mtiles = (long long)R / kSkinnyM + E;
+    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
+    dim3 grid((unsigned)(mtiles * ntile_n)), block(kSkinnyThreads);
+    if (elem_type == MOE_A2A_BF16)
+      return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_skinny_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
+                    (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+    return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_skinny_kernel<F16>, grid, block, 0, stream, (const uint4*)x,
+                  (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+  }
   const int ntile_n = ceil_div(N, kGemmN);
   // worst case of m-tiles: every expert ends with a partly filled tile
   const long long mtiles = (long long)R / kGemmM + E;

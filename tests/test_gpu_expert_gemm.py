@@ -44,9 +44,11 @@ def make(E, K, T, H, N, W, dtype, seed, zipf=False):
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-@pytest.mark.parametrize("tile", ["128", "256"], ids=["tile128", "tile256"])
+@pytest.mark.parametrize("tile", ["32", "128", "256"], ids=["tile32", "tile128", "tile256"])
 def test_expert_gemm_matches_f32_reference(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, padded, tile):
-    monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile)  # both kernels on every shape
+    # every kernel on every shape (the 32-row kernel needs H % 128 == 0; the library takes the
+    # 128 x 128 kernel for the other hidden sizes)
+    monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=E + T, zipf=zipf)
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, W, padded=padded, max_recv=T if padded else None)
@@ -62,7 +64,7 @@ def test_expert_gemm_matches_f32_reference(gpu_device, monkeypatch, E, K, T, H, 
 
 
 @pytest.mark.parametrize("E,K,T,H,N,zipf", [
-    (8, 2, 1200, 192, 264, False),   # 300 rows per expert: the library itself picks the 256 x 256 kernel
+    (8, 2, 1200, 384, 264, False),   # 300 rows per expert: the library itself picks the 256 x 256 kernel
     (16, 4, 1500, 256, 512, True),   # skewed, segments from empty to well past one tile
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
@@ -76,7 +78,7 @@ def test_both_tile_sizes_give_the_same_bits(gpu_device, monkeypatch, E, K, T, H,
     wd = weights.to(gpu_device)
     lib = ata.lib
     outs = {}
-    for tile in ("default", "128", "256"):
+    for tile in ("default", "32", "128", "256"):
         if tile == "default":
             monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
         else:
@@ -88,8 +90,9 @@ def test_both_tile_sizes_give_the_same_bits(gpu_device, monkeypatch, E, K, T, H,
         ids, us = (ctypes.c_int * 4)(), (ctypes.c_float * 4)()
         assert lib.moe_a2a_timer_end(ids, us, 4) == 1
         name = lib.moe_a2a_kernel_name(ids[0]).decode()
-        assert name == ("expert_gemm" if tile == "128" else "expert_gemm_wide")
+        assert name == {"32": "expert_gemm_skinny", "128": "expert_gemm"}.get(tile, "expert_gemm_wide")
     assert torch.equal(outs["128"].view(torch.int16), outs["256"].view(torch.int16))
+    assert torch.equal(outs["32"].view(torch.int16), outs["256"].view(torch.int16))
     assert torch.equal(outs["default"].view(torch.int16), outs["256"].view(torch.int16))
     o = V.run_world(cfg, world)
     close(outs["256"], V.expert_gemm(o["disp_x"], o["offsets"], weights, dtype))
@@ -133,6 +136,29 @@ def test_fp8_gemm_feeds_combine(gpu_device):
     ey = V.expert_gemm_fp8(o["disp_x"], o["disp_scale"], o["offsets"], weights, torch.bfloat16)
     want = V.combine_f32(ey, w.cpu(), o["slot_of_entry"], torch.bfloat16)
     close(y, want)
+
+
+def test_decode_shape_takes_the_skinny_kernel(gpu_device, monkeypatch):
+    """Eight rows per expert on average (the headline routing shape): the library picks the
+    32 x 256 kernel by itself, and its bits equal the 128 x 128 kernel's."""
+    monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
+    cfg, world, weights = make(256, 8, 256, 1024, 520, 8, torch.bfloat16, seed=11)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, 8)
+    d = ata.dispatch(x, idx, rs)
+    wd = weights.to(gpu_device)
+    import ctypes
+    assert ata.lib.moe_a2a_timer_begin(4) == 0
+    y = ata.expert_gemm(d, wd).clone()
+    torch.cuda.synchronize()
+    ids, us = (ctypes.c_int * 4)(), (ctypes.c_float * 4)()
+    assert ata.lib.moe_a2a_timer_end(ids, us, 4) == 1
+    assert ata.lib.moe_a2a_kernel_name(ids[0]) == b"expert_gemm_skinny"
+    monkeypatch.setenv("MOE_A2A_GEMM_TILE", "128")
+    y128 = ata.expert_gemm(d, wd)
+    assert torch.equal(y.view(torch.int16), y128.view(torch.int16))
+    o = V.run_world(cfg, world)
+    close(y, V.expert_gemm(o["disp_x"], o["offsets"], weights, torch.bfloat16))
 
 
 def test_dispatch_gemm_combine_end_to_end(gpu_device):
