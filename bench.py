@@ -328,8 +328,18 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
                config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N, kernel=kernel,
                            rows_dtype="fp8 e4m3fn + f32 scale per 128 columns" if fp8 else "16-bit"),
                kernels_us=summarise(per),
-               roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
-                             frac=round(tflops / MFMA_PEAK_TFLOPS, 4), traffic=None))
+               )
+    # which roof: the operands must cross HBM once (rows, the weights of every expert that has rows,
+    # the output); if that takes longer at 8 TB/s than the flops at the MFMA peak, the launch is HBM-bound
+    live = int((d.counts > 0).sum())
+    gemm_bytes = R * H * (1 + 4 / 128 if fp8 else 2) + live * N * H * 2 + R * N * 2
+    if gemm_bytes / (HBM_PEAK_GBPS * 1e3) > flops / (MFMA_PEAK_TFLOPS * 1e6):
+        gbps = gemm_bytes / t_us / 1e3
+        out["roofline"] = dict(bound="hbm", achieved=round(gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
+                               frac=round(gbps / HBM_PEAK_GBPS, 4), traffic=None)
+    else:
+        out["roofline"] = dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                               frac=round(tflops / MFMA_PEAK_TFLOPS, 4), traffic=None)
     if not args.no_cpu:
         from oracle import all2all_vec as O
 
