@@ -1117,8 +1117,8 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16_v<F16>(const u32x4_t& a, const
 // MFMAs are spent on rows that do not exist than with 128-row tiles), four waves side by side on
 // 32 x 32 each, K slabs of 128 (256 contiguous bytes of every weight row per slab: measured 6.09
 // TB/s of weights at 256 experts x 8 rows, 7168 -> 2048, against 5.95 with 256 x 64 slabs and 5.84
-// for the 128 x 128 kernel), and the global -> register prefetch runs TWO slabs ahead in two
-// register sets.  Accumulation order over K equals the other kernels': same bits.
+// for the 128 x 128 kernel), weights loaded non-temporally (each is read once: 6.65 TB/s), and the
+// global -> register prefetch runs TWO slabs ahead in two register sets.  Accumulation order over K equals the other kernels': same bits.
 constexpr int kSkinnyM = 32, kSkinnyThreads = 256;
 #ifndef MOE_A2A_SKINNY_N
 #define MOE_A2A_SKINNY_N 128
@@ -1196,7 +1196,7 @@ __global__ __launch_bounds__(kSkinnyThreads, 3) void expert_gemm_skinny_kernel(c
   {                                                                            \
     const int kv_ = min((K0), Kd - BK) >> 3; /* past the end: the last slab again */ \
     _Pragma("unroll") for (int i = 0; i < NA; ++i) RA[i] = xa[offa[i] + kv_];  \
-    _Pragma("unroll") for (int i = 0; i < NB; ++i) RB[i] = wb[offb[i] + kv_];  \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) RB[i] = __builtin_nontemporal_load(wb + offb[i] + kv_); \
   }
 #define SKINNY_STASH(RA, RB)                                                                          \
   {                                                                                                   \
