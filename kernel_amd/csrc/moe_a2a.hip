@@ -34,9 +34,12 @@ constexpr int kRouteTilesMaxRows = 16 * kRouteThreads;  // one-launch routing up
 constexpr int kRowMaxThreads = 512;
 constexpr int kFusedIdBits = 13;
 constexpr int kFusedMaxRows = 1 << kFusedIdBits;  // route_dispatch packs (expert, entry id) into one key
-constexpr int kFusedEntriesPerThread = 4;
+constexpr int kFusedMaxEntriesPerThread = 32;
 constexpr int kFusedMaxThreads = 1024;
-constexpr long long kFusedMaxTableReads = 1ll << 20;  // entries read by all workgroups together
+#ifndef MOE_A2A_FUSED_TABLE_READS
+#define MOE_A2A_FUSED_TABLE_READS (1ll << 23)
+#endif
+constexpr long long kFusedMaxTableReads = MOE_A2A_FUSED_TABLE_READS;  // entries read by all workgroups together
 
 enum KernelId {
   KID_ROUTE_TILES = 0,
@@ -477,11 +480,12 @@ __global__ __launch_bounds__(kRowMaxThreads) void dispatch_rows_kernel(const uin
 
 // Routing folded into the dispatch for R <= kFusedMaxRows.  The slot of entry i is the number
 // of entries whose (expert, entry id) pair is smaller, so a workgroup can find the K slots of
-// its own token by comparing every entry of the table against K keys: each lane holds
-// kFusedEntriesPerThread entries, a ballot + popcount per (entry, key) counts a wave's share,
+// its own token by comparing every entry of the table against K keys: each lane holds EPT
+// entries (all loaded in one go), a ballot + popcount per (entry, key) counts a wave's share,
 // and LDS counters add the waves up.  The row load is issued first and is in flight meanwhile.
 // Column split 0 of each token also writes the index arrays and meta rows; workgroup 0
 // writes counts and offsets.
+template <int EPT, bool PAD>  // EPT table entries per thread: 4 (small tables), 8, 16, 24 or 32; PAD: padded layout
 __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteArgs a, const uint4* __restrict__ x,
                                                                          uint4* __restrict__ disp, int nvec,
                                                                          int per, int nsplit) {
@@ -518,26 +522,37 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
   const int cs = (blockIdx.x - 1) - t * nsplit;
   const int c = cs * per + tid;
   const bool active = tid < per && c < nvec;
-  const int chunk = nthreads * kFusedEntriesPerThread;
-
-  // Raw expert ids of this lane's entries of the chunk starting at i0.  Indices are clamped
+  // Raw expert ids of this lane's entries.  EPT == 4: entries 4 tid .. 4 tid + 3, indices clamped
   // into the table instead of branching, like every load below: with unconditional loads the
-  // compiler can wait for the early ones while the later ones stay in flight.
-  int raw[kFusedEntriesPerThread];
-  auto load_chunk = [&](int i0) {
-    const int ibase = i0 + tid * kFusedEntriesPerThread;
-#pragma unroll
-    for (int m = 0; m < kFusedEntriesPerThread; ++m) raw[m] = a.indices[min(ibase + m, a.R - 1)];
-  };
-
-  // Counters are cleared and the barrier taken while nothing is in flight.  Then every load
-  // goes out before the first use of a loaded value: the first chunk of the table, the token's
-  // own expert ids (lane k of every wave holds entry k), the rank boundaries, and last the row
-  // itself, so that waiting for the indices (memory operations complete in order) leaves the
-  // row in flight while the slots are worked out.
+  // compiler can wait for the early ones while the later ones stay in flight.  Larger tables:
+  // EPT / 4 vectors of four entries, vector c at entry 4 (c nthreads + tid), all issued at once
+  // (one table round trip, not one per chunk); a vector that would cross the end of the table is
+  // moved back to end at the last entry, and the entries it then shares with its neighbour are
+  // masked out below.
+  // Counters are cleared and the barrier taken while nothing is in flight.
   if (tid < a.K) s_slot[tid] = 0;
   __syncthreads();
-  load_chunk(0);
+  int raw[EPT];
+  int pos[EPT / 4];
+  if (EPT == 4) {
+    pos[0] = tid * 4;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) raw[m] = a.indices[min(pos[0] + m, a.R - 1)];
+  } else {
+    typedef int i32x4_t __attribute__((ext_vector_type(4), aligned(4)));  // a moved vector is only dword-aligned
+#pragma unroll
+    for (int ch = 0; ch < EPT / 4; ++ch) {
+      pos[ch] = min((ch * nthreads + tid) * 4, a.R - 4);  // R >= 4 on this path
+      const i32x4_t q = *reinterpret_cast<const i32x4_t*>(a.indices + pos[ch]);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) raw[4 * ch + m] = q[m];
+    }
+  }
+
+  // Every load goes out before the first use of a loaded value: the table, the token's own expert ids
+  // (lane k of every wave holds entry k), the rank boundaries, and last the row itself, so that
+  // waiting for the indices (memory operations complete in order) leaves the row in flight while
+  // the slots are worked out.
   const int own = a.indices[t * a.K + min(lane, a.K - 1)];
   const bool want_starts = cs == 0 && a.rank_start != nullptr;
   const int32_t* sp = a.rank_start ? a.rank_start : a.indices;  // any readable address when unused
@@ -554,28 +569,30 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
     return (min(max(e, 0), a.E - 1) << kFusedIdBits) | i;
   };
   const int ownkey = lane < a.K ? key_of(own, t * a.K + lane) : 0x7fffffff;
-  // one chunk: count, for each of the token's K keys, the smaller keys this wave holds
-  auto count_chunk = [&](int i0) {
-    const int ibase = i0 + tid * kFusedEntriesPerThread;
-    int key[kFusedEntriesPerThread];
+  // count, for each of the token's K keys, the smaller keys this wave holds
+  int key[EPT];
 #pragma unroll
-    for (int m = 0; m < kFusedEntriesPerThread; ++m) key[m] = ibase + m < a.R ? key_of(raw[m], ibase + m) : 0x7fffffff;
-    if (__ballot(ibase < a.R) == 0) return;  // this wave holds no entries of the chunk
-    for (int k = 0; k < a.K; ++k) {
-      // compact: keys below mine; padded: keys below mine of my own expert (position in segment)
-      const unsigned mykey = (unsigned)__builtin_amdgcn_readlane(ownkey, k);
-      const unsigned lo = a.pad ? (mykey & ~((1u << kFusedIdBits) - 1u)) : 0u;
-      const unsigned span = mykey - lo;
-      int cnt = 0;
+  for (int ch = 0; ch < EPT / 4; ++ch) {
+    const int first = EPT == 4 ? pos[0] : (ch * nthreads + tid) * 4;  // first entry this vector owns
 #pragma unroll
-      for (int m = 0; m < kFusedEntriesPerThread; ++m) cnt += __popcll(__ballot((unsigned)key[m] - lo < span));
-      if (lane == 0 && cnt) atomicAdd(&s_slot[k], cnt);
+    for (int m = 0; m < 4; ++m) {
+      const int i = pos[ch] + m;
+      key[4 * ch + m] = (i >= first && i < a.R) ? key_of(raw[4 * ch + m], i) : 0x7fffffff;
     }
-  };
-  count_chunk(0);  // outside the loop: only here are the row and rank loads still in flight
-  for (int i0 = chunk; i0 < a.R; i0 += chunk) {
-    load_chunk(i0);
-    count_chunk(i0);
+  }
+  for (int k = 0; k < a.K; ++k) {
+    // compact: keys below mine; padded: keys below mine of my own expert (position in segment)
+    const unsigned mykey = (unsigned)__builtin_amdgcn_readlane(ownkey, k);
+    int cnt = 0;
+    if (PAD) {
+      const unsigned lo = mykey & ~((1u << kFusedIdBits) - 1u), span = mykey - lo;
+#pragma unroll
+      for (int m = 0; m < EPT; ++m) cnt += __popcll(__ballot((unsigned)key[m] - lo < span));
+    } else {  // one compare per (entry, key): this loop is the kernel's arithmetic
+#pragma unroll
+      for (int m = 0; m < EPT; ++m) cnt += __popcll(__ballot((unsigned)key[m] < mykey));
+    }
+    if (lane == 0 && cnt) atomicAdd(&s_slot[k], cnt);
   }
   if (bad && a.status) *a.status = 1;
   if (want_starts) {  // W + 1 <= 257 <= 2 * nthreads
@@ -584,7 +601,7 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
   }
   __syncthreads();
 
-  if (a.pad) {  // position in segment -> row of the padded layout (counts are final here)
+  if (PAD) {  // position in segment -> row of the padded layout (counts are final here)
     if (tid < a.K) s_slot[tid] = row_of(a, ownkey >> kFusedIdBits, s_slot[tid], 0);
     __syncthreads();
   }
@@ -1663,12 +1680,21 @@ int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, 
 
 int moe_a2a_fused_max_rows(void) { return kFusedMaxRows; }
 
+// Table entries each thread of the fused kernel holds: the smallest of 4, 8, 16, 24, 32 that covers
+// R entries with `threads` threads, 0 when even 32 do not.
+static int fused_entries_per_thread(int R, int threads) {
+  for (int ept : {4, 8, 16, 24, 32})
+    if ((long long)threads * ept >= R) return ept;
+  return 0;
+}
+
 int moe_a2a_fused_ok(int T, int K, int H) {
   if (T < 1 || K < 1 || H < 8) return 0;
   const long long R = (long long)T * K;
   if (R > kFusedMaxRows) return 0;
   const RowGeom g = row_geom(H / 8, 1, kFusedMaxThreads, 256);
-  // every workgroup reads the whole routing table: keep that traffic far below the payload
+  if (fused_entries_per_thread((int)R, g.threads) == 0) return 0;
+  // every workgroup reads the whole routing table (from L2): keep that traffic below the payload
   return R * T * g.nsplit <= kFusedMaxTableReads ? 1 : 0;
 }
 
@@ -1686,8 +1712,23 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
               slot_of_entry, src_of_slot, meta, status};
   const int nvec = H / 8;
   const RowGeom g = row_geom(nvec, 1, kFusedMaxThreads, 256);
-  return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel, dim3((unsigned)T * g.nsplit + 1), dim3(g.threads), 0,
-                (hipStream_t)stream_, a, (const uint4*)x, (uint4*)disp_x, nvec, g.per, g.nsplit);
+  const int ept = fused_entries_per_thread(T * K, g.threads);
+  if (ept == 0) return MOE_A2A_E_SHAPE;
+  dim3 grid((unsigned)T * g.nsplit + 1), block(g.threads);
+#define CALL_FUSED(EPT)                                                                                        \
+  {                                                                                                            \
+    if (max_recv > 0)                                                                                          \
+      return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<EPT, true>, grid, block, 0, (hipStream_t)stream_, a, \
+                    (const uint4*)x, (uint4*)disp_x, nvec, g.per, g.nsplit);                                   \
+    return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<EPT, false>, grid, block, 0, (hipStream_t)stream_, a, \
+                  (const uint4*)x, (uint4*)disp_x, nvec, g.per, g.nsplit);                                     \
+  }
+  if (ept == 4) CALL_FUSED(4);
+  if (ept == 8) CALL_FUSED(8);
+  if (ept == 16) CALL_FUSED(16);
+  if (ept == 24) CALL_FUSED(24);
+  CALL_FUSED(32);
+#undef CALL_FUSED
 }
 
 int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry, uint8_t* disp_q,
