@@ -489,7 +489,7 @@ template <int EPT, bool PAD>  // EPT table entries per thread: 4 (small tables),
 __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteArgs a, const uint4* __restrict__ x,
                                                                          uint4* __restrict__ disp, int nvec,
                                                                          int per, int nsplit) {
-  __shared__ int s_slot[MOE_A2A_MAX_TOPK];
+  __shared__ int s_part[kFusedMaxThreads / kWave][MOE_A2A_MAX_TOPK];  // per wave: smaller keys it holds, per key
   __shared__ int s_hist[MOE_A2A_MAX_EXPERTS];
   __shared__ int s_tmp[kFusedMaxThreads / kWave + 1];
   __shared__ int s_starts[MOE_A2A_MAX_WORLD + 1];
@@ -529,9 +529,6 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
   // (one table round trip, not one per chunk); a vector that would cross the end of the table is
   // moved back to end at the last entry, and the entries it then shares with its neighbour are
   // masked out below.
-  // Counters are cleared and the barrier taken while nothing is in flight.
-  if (tid < a.K) s_slot[tid] = 0;
-  __syncthreads();
   int raw[EPT];
   int pos[EPT / 4];
   if (EPT == 4) {
@@ -592,7 +589,7 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
 #pragma unroll
       for (int m = 0; m < EPT; ++m) cnt += __popcll(__ballot((unsigned)key[m] < mykey));
     }
-    if (lane == 0 && cnt) atomicAdd(&s_slot[k], cnt);
+    if (lane == 0) s_part[tid / kWave][k] = cnt;  // plain stores: nothing to clear, one barrier in all
   }
   if (bad && a.status) *a.status = 1;
   if (want_starts) {  // W + 1 <= 257 <= 2 * nthreads
@@ -601,15 +598,20 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
   }
   __syncthreads();
 
-  if (PAD) {  // position in segment -> row of the padded layout (counts are final here)
-    if (tid < a.K) s_slot[tid] = row_of(a, ownkey >> kFusedIdBits, s_slot[tid], 0);
-    __syncthreads();
+  // every wave adds the partial counts up for itself: lane k takes key k, lane reads hand the K
+  // slots round (no second barrier, no shared result)
+  int myslot = 0;
+  if (lane < a.K) {
+    const int nwaves = (nthreads + kWave - 1) / kWave;
+    for (int wv = 0; wv < nwaves; ++wv) myslot += s_part[wv][lane];
+    if (PAD) myslot = row_of(a, ownkey >> kFusedIdBits, myslot, 0);  // position in segment -> padded row
   }
   if (active)
-    for (int k = 0; k < a.K; ++k) store_through(disp + (size_t)s_slot[k] * nvec + c, v);
+    for (int k = 0; k < a.K; ++k)
+      store_through(disp + (size_t)__builtin_amdgcn_readlane(myslot, k) * nvec + c, v);
   if (cs == 0 && tid < a.K) {
     const int i = t * a.K + tid;
-    const int slot = s_slot[tid];
+    const int slot = myslot;
     a.slot_of_entry[i] = slot;
     a.src_of_slot[slot] = i;
     int sr, tl;
