@@ -773,6 +773,7 @@ struct EntryLanes {
   float w;    // lane k: routing weight of entry k
   float f;    // lane k: stub factor of entry k (stub_combine only)
   int pos;    // lane k: position of entry k in the fold order
+  int src;    // lane j: the lane whose entry has fold position j
   bool live;  // lane < K
 };
 
@@ -790,12 +791,16 @@ __device__ __forceinline__ EntryLanes load_entries(const int32_t* __restrict__ s
     en.w = weights[(size_t)t * K + lane];
   }
   en.pos = lane;
+  en.src = lane;
   if (MODE == MOE_A2A_COMBINE_STRICT) {
     en.pos = 0;
     for (int j = 0; j < K; ++j) {
       const int sj = __builtin_amdgcn_readlane(en.slot, j);
       en.pos += sj < en.slot || (sj == en.slot && j < lane);  // ties by k keep positions distinct
     }
+    // invert the permutation with one cross-lane scatter: lane pos receives this lane's number
+    // (lanes >= K all land on lane K, which nobody reads)
+    en.src = __builtin_amdgcn_ds_permute(en.pos << 2, lane);
   }
   return en;
 }
@@ -809,7 +814,7 @@ __device__ __forceinline__ float lane_read(float x, int src) {
 template <int MODE>
 __device__ __forceinline__ int entry_lane(const EntryLanes& en, int j) {
   if (MODE != MOE_A2A_COMBINE_STRICT) return j;
-  return __builtin_amdgcn_readfirstlane(__ffsll((long long)__ballot(en.live && en.pos == j)) - 1);
+  return __builtin_amdgcn_readlane(en.src, j);
 }
 
 template <class E, int MODE>
