@@ -485,7 +485,10 @@ __global__ __launch_bounds__(kRowMaxThreads) void dispatch_rows_kernel(const uin
 // and LDS counters add the waves up.  The row load is issued first and is in flight meanwhile.
 // Column split 0 of each token also writes the index arrays and meta rows; workgroup 0
 // writes counts and offsets.
-template <int EPT, bool PAD>  // EPT table entries per thread: 4 (small tables), 8, 16, 24 or 32; PAD: padded layout
+// EPT table entries per thread: 4 (small tables), 8, 16, 24 or 32; PAD: padded layout; VPL row
+// vectors per lane: 2 for long rows (half as many waves to launch: 7.4 against 7.6 us at 256 tokens
+// of 7168 columns), 1 otherwise (two were slower at 2048 columns, four at both).
+template <int EPT, bool PAD, int VPL>
 __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteArgs a, const uint4* __restrict__ x,
                                                                          uint4* __restrict__ disp, int nvec,
                                                                          int per, int nsplit) {
@@ -520,8 +523,13 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
 
   const int t = (blockIdx.x - 1) / nsplit;
   const int cs = (blockIdx.x - 1) - t * nsplit;
-  const int c = cs * per + tid;
-  const bool active = tid < per && c < nvec;
+  int cv[VPL];
+  bool active[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    cv[j] = (cs * VPL + j) * per + tid;
+    active[j] = tid < per && cv[j] < nvec;
+  }
   // Raw expert ids of this lane's entries.  EPT == 4: entries 4 tid .. 4 tid + 3, indices clamped
   // into the table instead of branching, like every load below: with unconditional loads the
   // compiler can wait for the early ones while the later ones stay in flight.  Larger tables:
@@ -556,7 +564,9 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
   const int st0 = sp[a.rank_start ? min(tid, a.W) : 0];
   const int st1 = sp[a.rank_start ? min(tid + nthreads, a.W) : 0];
   __builtin_amdgcn_sched_barrier(0);  // keep the row load behind the index loads
-  const uint4 v = x[(size_t)t * nvec + min(c, nvec - 1)];
+  uint4 v[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) v[j] = x[(size_t)t * nvec + min(cv[j], nvec - 1)];
   __builtin_amdgcn_sched_barrier(0);
 
   // ids outside [0, E) are clamped without branching; one flag store at the end reports them
@@ -606,9 +616,12 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
     for (int wv = 0; wv < nwaves; ++wv) myslot += s_part[wv][lane];
     if (PAD) myslot = row_of(a, ownkey >> kFusedIdBits, myslot, 0);  // position in segment -> padded row
   }
-  if (active)
-    for (int k = 0; k < a.K; ++k)
-      store_through(disp + (size_t)__builtin_amdgcn_readlane(myslot, k) * nvec + c, v);
+  for (int k = 0; k < a.K; ++k) {
+    uint4* row = disp + (size_t)__builtin_amdgcn_readlane(myslot, k) * nvec;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      if (active[j]) store_through(row + cv[j], v[j]);
+  }
   if (cs == 0 && tid < a.K) {
     const int i = t * a.K + tid;
     const int slot = myslot;
@@ -1687,6 +1700,12 @@ int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, 
 
 int moe_a2a_fused_max_rows(void) { return kFusedMaxRows; }
 
+// Geometry of the fused kernel: lanes of a workgroup and row vectors per lane.
+static int fused_vectors_per_lane(int nvec) { return nvec >= 768 ? 2 : 1; }
+static RowGeom fused_geom(int nvec) {
+  return row_geom(ceil_div(nvec, fused_vectors_per_lane(nvec)), 1, kFusedMaxThreads, 256);
+}
+
 // Table entries each thread of the fused kernel holds: the smallest of 4, 8, 16, 24, 32 that covers
 // R entries with `threads` threads, 0 when even 32 do not.
 static int fused_entries_per_thread(int R, int threads) {
@@ -1699,7 +1718,7 @@ int moe_a2a_fused_ok(int T, int K, int H) {
   if (T < 1 || K < 1 || H < 8) return 0;
   const long long R = (long long)T * K;
   if (R > kFusedMaxRows) return 0;
-  const RowGeom g = row_geom(H / 8, 1, kFusedMaxThreads, 256);
+  const RowGeom g = fused_geom(H / 8);
   if (fused_entries_per_thread((int)R, g.threads) == 0) return 0;
   // every workgroup reads the whole routing table (from L2): keep that traffic below the payload
   return R * T * g.nsplit <= kFusedMaxTableReads ? 1 : 0;
@@ -1718,23 +1737,29 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
               slot_of_entry, src_of_slot, meta, status};
   const int nvec = H / 8;
-  const RowGeom g = row_geom(nvec, 1, kFusedMaxThreads, 256);
+  const RowGeom g = fused_geom(nvec);
+  const int vpl = fused_vectors_per_lane(nvec);
   const int ept = fused_entries_per_thread(T * K, g.threads);
   if (ept == 0) return MOE_A2A_E_SHAPE;
   dim3 grid((unsigned)T * g.nsplit + 1), block(g.threads);
+#define CALL_FUSED3(EPT, PAD, VPL)                                                                             \
+  return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<EPT, PAD, VPL>, grid, block, 0, (hipStream_t)stream_, a, \
+                (const uint4*)x, (uint4*)disp_x, nvec, g.per, g.nsplit)
 #define CALL_FUSED(EPT)                                                                                        \
   {                                                                                                            \
-    if (max_recv > 0)                                                                                          \
-      return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<EPT, true>, grid, block, 0, (hipStream_t)stream_, a, \
-                    (const uint4*)x, (uint4*)disp_x, nvec, g.per, g.nsplit);                                   \
-    return launch(KID_ROUTE_DISPATCH, route_dispatch_kernel<EPT, false>, grid, block, 0, (hipStream_t)stream_, a, \
-                  (const uint4*)x, (uint4*)disp_x, nvec, g.per, g.nsplit);                                     \
+    if (max_recv > 0) {                                                                                        \
+      if (vpl == 2) CALL_FUSED3(EPT, true, 2);                                                                 \
+      CALL_FUSED3(EPT, true, 1);                                                                               \
+    }                                                                                                          \
+    if (vpl == 2) CALL_FUSED3(EPT, false, 2);                                                                  \
+    CALL_FUSED3(EPT, false, 1);                                                                                \
   }
   if (ept == 4) CALL_FUSED(4);
   if (ept == 8) CALL_FUSED(8);
   if (ept == 16) CALL_FUSED(16);
   if (ept == 24) CALL_FUSED(24);
   CALL_FUSED(32);
+#undef CALL_FUSED3
 #undef CALL_FUSED
 }
 
