@@ -123,7 +123,7 @@ def summarise(per):
 
 
 ROUTE_KERNELS = ("route_tiles", "route_hist", "route_scan", "route_rank")
-DISPATCH_KERNELS = ("dispatch_rows", "route_dispatch", "dispatch_fp8")
+DISPATCH_KERNELS = ("dispatch_rows", "route_dispatch", "route_dispatch_tile", "dispatch_fp8")
 COMBINE_KERNELS = ("combine_rows", "stub_combine")
 STUB_KERNELS = ("stub_rows", "stub_fp8")
 

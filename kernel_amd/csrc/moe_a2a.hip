@@ -21,6 +21,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <algorithm>
 #include <atomic>
 
 #include "moe_a2a.h"
@@ -37,7 +38,7 @@ constexpr int kFusedMaxRows = 1 << kFusedIdBits;  // route_dispatch packs (exper
 constexpr int kFusedMaxEntriesPerThread = 32;
 constexpr int kFusedMaxThreads = 1024;
 #ifndef MOE_A2A_FUSED_TABLE_READS
-#define MOE_A2A_FUSED_TABLE_READS (1ll << 23)
+#define MOE_A2A_FUSED_TABLE_READS (1ll << 20)
 #endif
 constexpr long long kFusedMaxTableReads = MOE_A2A_FUSED_TABLE_READS;  // entries read by all workgroups together
 
@@ -48,6 +49,7 @@ enum KernelId {
   KID_ROUTE_RANK,
   KID_DISPATCH,
   KID_ROUTE_DISPATCH,
+  KID_ROUTE_DISPATCH_TILE,
   KID_DISPATCH_FP8,
   KID_STUB,
   KID_STUB_FP8,
@@ -59,7 +61,7 @@ enum KernelId {
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
-    "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch",
+    "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
     "expert_gemm_wide", "expert_gemm_skinny"};
 
@@ -635,6 +637,97 @@ __global__ __launch_bounds__(kFusedMaxThreads) void route_dispatch_kernel(RouteA
     m[2] = tl;
     m[3] = tid;
     m[4] = 0;
+  }
+}
+
+// Routing + dispatch in ONE launch for any table size.  A workgroup owns a tile of consecutive
+// tokens.  It histograms the whole routing table once into two LDS rows per expert (entries before
+// the tile / from the tile on), scans the experts for the segment starts, ranks its own entries
+// (at most kTileMaxOwn) against each other, and then copies its tokens' rows, a batch of vectors
+// per thread at a time; the first batch of row loads is issued before the routing so that it is in
+// flight meanwhile.  The table pass costs O(R / threads) per workgroup and is amortised over the
+// tile's tokens, where the one-token kernel above pays O(R K / threads) per token.  Counts are
+// integer sums: the result does not depend on the order of the LDS atomics.
+constexpr int kTileThreads = 1024;
+constexpr int kTileMaxOwn = 256;  // entries (tokens * K) of a tile
+constexpr int kTileBatch = 4;     // row vectors per thread and batch
+
+template <int STREAM>
+__global__ __launch_bounds__(kTileThreads) void route_dispatch_tile_kernel(RouteArgs a, const uint4* __restrict__ x,
+                                                                          uint4* __restrict__ disp, int nvec,
+                                                                          int tile_tokens) {
+  __shared__ int s_cnt[2 * MOE_A2A_MAX_EXPERTS];  // [0,E): entries before the tile, [E,2E): the rest
+  __shared__ int s_base[MOE_A2A_MAX_EXPERTS];     // compact slot of the tile's first entry of each expert
+  __shared__ int s_tmp[kTileThreads / kWave + 1];
+  __shared__ int s_starts[MOE_A2A_MAX_WORLD + 1];
+  __shared__ int s_own[kTileMaxOwn];   // expert of each entry of the tile
+  __shared__ int s_slot[kTileMaxOwn];  // its destination row
+  const int tid = threadIdx.x;
+  const int t0 = blockIdx.x * tile_tokens;
+  const int ntok = min(tile_tokens, a.T - t0);
+  const int first = t0 * a.K, n_own = ntok * a.K;
+  const int items = ntok * nvec;  // row vectors of the tile; the tile's rows are contiguous in x
+  const uint4* xt = x + (size_t)t0 * nvec;
+
+  uint4 v[kTileBatch];
+#pragma unroll
+  for (int b = 0; b < kTileBatch; ++b) v[b] = load_row<STREAM>(xt + min(tid + b * kTileThreads, items - 1));
+
+  for (int j = tid; j < 2 * a.E; j += kTileThreads) s_cnt[j] = 0;
+  load_starts(a, s_starts);
+  __syncthreads();
+  for (int i0 = 0; i0 < a.R; i0 += 4 * kTileThreads) {  // four loads in flight per thread
+    int e[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) e[m] = a.indices[min(i0 + m * kTileThreads + tid, a.R - 1)];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int i = i0 + m * kTileThreads + tid;
+      if (i < a.R) atomicAdd(&s_cnt[(i < first ? 0 : a.E) + clamp_expert(a, e[m])], 1);
+    }
+  }
+  __syncthreads();
+  const int all = tid < a.E ? s_cnt[tid] + s_cnt[a.E + tid] : 0;
+  int total;
+  const int run = block_exclusive_scan(all, s_tmp, total);
+  if (tid < a.E) {
+    s_base[tid] = run + s_cnt[tid];
+    if (blockIdx.x == 0) {
+      a.counts[tid] = all;
+      a.offsets[tid] = run;
+    }
+  }
+  if (blockIdx.x == 0 && tid == 0) a.offsets[a.E] = total;
+  int e_own = 0;
+  if (tid < n_own) {
+    e_own = load_expert(a, first + tid, true);
+    s_own[tid] = e_own;
+  }
+  __syncthreads();
+  if (tid < n_own) {
+    int rank = 0;  // earlier entries of the tile with the same expert (every lane reads the same word)
+    for (int j = 0; j < tid; ++j) rank += s_own[j] == e_own;
+    const int first_of_e = s_base[e_own] - s_cnt[e_own];
+    const int slot = s_base[e_own] + rank;
+    emit_entry(a, s_starts, first + tid, e_own, slot, first_of_e);
+    s_slot[tid] = row_of(a, e_own, slot, first_of_e);
+  }
+  __syncthreads();
+
+  for (int base = 0; base < items; base += kTileBatch * kTileThreads) {
+    if (base > 0) {
+#pragma unroll
+      for (int b = 0; b < kTileBatch; ++b) v[b] = load_row<STREAM>(xt + min(base + tid + b * kTileThreads, items - 1));
+    }
+#pragma unroll
+    for (int b = 0; b < kTileBatch; ++b) {
+      const int item = base + tid + b * kTileThreads;
+      if (item < items) {
+        const int tt = item / nvec;
+        const int c = item - tt * nvec;
+        for (int k = 0; k < a.K; ++k) store_row<STREAM>(disp + (size_t)s_slot[tt * a.K + k] * nvec + c, v[b]);
+      }
+    }
   }
 }
 
@@ -1698,7 +1791,7 @@ int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, 
                 slot_of_entry, (uint4*)disp_x, K, nvec, g.per, g.nsplit);
 }
 
-int moe_a2a_fused_max_rows(void) { return kFusedMaxRows; }
+int moe_a2a_fused_max_rows(void) { return INT32_MAX / 8; }
 
 // Geometry of the fused kernel: lanes of a workgroup and row vectors per lane.
 static int fused_vectors_per_lane(int nvec) { return nvec >= 768 ? 2 : 1; }
@@ -1719,14 +1812,34 @@ static int fused_entries_per_thread(int R, int threads) {
   return 0;
 }
 
-int moe_a2a_fused_ok(int T, int K, int H) {
-  if (T < 1 || K < 1 || H < 8) return 0;
+// The one-token-per-workgroup kernel: small tables only.
+static bool fused_small_ok(int T, int K, int H) {
+  if (T < 1 || K < 1 || H < 8) return false;
   const long long R = (long long)T * K;
-  if (R > kFusedMaxRows) return 0;
+  if (R > kFusedMaxRows) return false;
   const RowGeom g = fused_geom(H / 8, (int)R);
-  if (fused_entries_per_thread((int)R, g.threads) == 0) return 0;
+  if (fused_entries_per_thread((int)R, g.threads) == 0) return false;
   // every workgroup reads the whole routing table (from L2): keep that traffic below the payload
-  return R * T * g.nsplit <= kFusedMaxTableReads ? 1 : 0;
+  return R * T * g.nsplit <= kFusedMaxTableReads;
+}
+
+// Tokens per workgroup of the tile kernel: at most kTileMaxOwn entries per tile; enough tokens that
+// the table passes of all workgroups together read at most a quarter of the bytes the dispatch
+// writes ((T / tile) * R * 4 <= R * H * 2 / 4, i.e. tile >= 8 T / H); otherwise as few as possible
+// (more workgroups).
+static int tile_tokens(int T, int K, int H) {
+  const int cap = kTileMaxOwn / K > 0 ? kTileMaxOwn / K : 1;
+  int tile = ceil_div((int)std::min<long long>(8ll * T, INT32_MAX), H);
+  if (tile < 1) tile = 1;
+  return tile < cap ? tile : cap;
+}
+
+int moe_a2a_fused_ok(int T, int K, int H) {
+  if (T < 1 || K < 1 || K > kTileMaxOwn || H < 8) return 0;
+  if (fused_small_ok(T, K, H)) return 1;
+  // Token tiles pay off while the rows stay cache-resident (measured: 26 against 35 us at 134 MB of
+  // rows, 151 against 110 us at 537 MB); the streaming sizes keep separate routing and dispatch.
+  return streams(T, (long long)T * K, H, 2, 2) ? 0 : 1;
 }
 
 int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
@@ -1735,13 +1848,24 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
                            void* disp_x, moe_a2a_stream_t stream_) {
   if (int rc = check_route_shape(T, K, E, W)) return rc;
   if (max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
-  if ((long long)T * K > kFusedMaxRows) return MOE_A2A_E_SHAPE;
   if (int rc = check_rows(x, disp_x, T, K, H, 8)) return rc;
   if (!counts || !offsets) return MOE_A2A_E_NULL;
   if (T > 0 && (!indices || !slot_of_entry || !src_of_slot || !meta)) return MOE_A2A_E_NULL;
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
               slot_of_entry, src_of_slot, meta, status};
   const int nvec = H / 8;
+  const char* force_tile = getenv("MOE_A2A_ROUTE_TILE");  // tuning aid: 1 forces the token-tile kernel
+  if (!fused_small_ok(T, K, H) || (force_tile && atoi(force_tile) == 1)) {  // token tiles: any table size
+    if (T == 0) return moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets,
+                                     slot_of_entry, src_of_slot, meta, status, nullptr, 0, stream_);
+    const int tile = tile_tokens(T, K, H);
+    dim3 grid((unsigned)ceil_div(T, tile)), block(kTileThreads);
+    if (streams(T, (long long)T * K, H, 2, 2))
+      return launch(KID_ROUTE_DISPATCH_TILE, route_dispatch_tile_kernel<1>, grid, block, 0, (hipStream_t)stream_, a,
+                    (const uint4*)x, (uint4*)disp_x, nvec, tile);
+    return launch(KID_ROUTE_DISPATCH_TILE, route_dispatch_tile_kernel<0>, grid, block, 0, (hipStream_t)stream_, a,
+                  (const uint4*)x, (uint4*)disp_x, nvec, tile);
+  }
   const RowGeom g = fused_geom(nvec, T * K);
   const int vpl = fused_vectors_per_lane(nvec);
   const int ept = fused_entries_per_thread(T * K, g.threads);
@@ -1978,8 +2102,7 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   if (!known_type(in_type) || !known_type(out_type)) return MOE_A2A_E_DTYPE;
   if (fp8_dispatch && !disp_scale) return MOE_A2A_E_NULL;
   if (!fuse_stub && T > 0 && !expert_y) return MOE_A2A_E_NULL;
-  const bool fused = !fp8_dispatch && (fuse_route == 2 ? (T > 0 && (long long)T * K <= kFusedMaxRows)
-                                                         : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
+  const bool fused = !fp8_dispatch && T > 0 && (fuse_route == 2 || fuse_route == 1) && moe_a2a_fused_ok(T, K, H);
   if (fused) {
     if (int rc = moe_a2a_route_dispatch(x, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts, offsets,
                                         slot_of_entry, src_of_slot, meta, status, disp, stream))

@@ -55,8 +55,9 @@ def test_version_strings_and_queries(lib):
     assert lib.moe_a2a_fused_max_rows() >= 2048
     assert lib.moe_a2a_fused_ok(256, 8, 7168) == 1  # the headline shape takes the one-launch path
     assert lib.moe_a2a_fused_ok(16384, 4, 4096) == 0
-    assert lib.moe_a2a_fused_ok(1024, 6, 2048) == 1  # 24 table entries per thread, one table round trip
-    assert lib.moe_a2a_fused_ok(2048, 4, 2048) == 0  # 16.8 M table entries read: more than the payload is worth
+    assert lib.moe_a2a_fused_ok(1024, 6, 2048) == 1  # mid-size table: one launch with token tiles
+    assert lib.moe_a2a_fused_ok(2048, 4, 2048) == 1
+    assert lib.moe_a2a_fused_ok(4096, 8, 7168) == 0  # streaming sizes keep separate routing and dispatch
 
 
 def test_route_rejects_bad_arguments(lib):
