@@ -109,13 +109,15 @@ int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, 
                      moe_a2a_stream_t stream);
 
 /*
- * Routing and dispatch in ONE launch for small worlds (R = T*K <= moe_a2a_fused_max_rows()):
- * every workgroup derives the slots of its own token from the routing table, so no
- * routing kernel has to finish first.  Outputs as moe_a2a_route + moe_a2a_dispatch.
+ * Routing and dispatch in ONE launch: every workgroup derives the slots of its own tokens from
+ * the routing table, so no routing kernel has to finish first and no workspace is needed.
+ * Outputs as moe_a2a_route + moe_a2a_dispatch.  Two kernels behind it: one token per workgroup
+ * for small tables, a tile of tokens per workgroup (at most 256 entries, so K <= 256) otherwise;
+ * any table size is accepted.
  */
-int moe_a2a_fused_max_rows(void);
-/* 1 if moe_a2a_route_dispatch is the faster choice for this shape: it needs R within the limit
- * above and a routing table small enough that re-reading it in every workgroup stays cheap. */
+int moe_a2a_fused_max_rows(void); /* largest R = T*K the one-launch form takes */
+/* 1 if moe_a2a_route_dispatch is the faster choice for this shape: always for cache-resident
+ * sizes; at streaming sizes (more than ~192 MB moved) separate routing and dispatch win. */
 int moe_a2a_fused_ok(int T, int K, int H);
 int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
                            int K, int E, int W, int H, int max_recv, int32_t* counts, int32_t* offsets,
@@ -168,7 +170,7 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
  * one host call keeps the launches back to back.
  *   fp8_dispatch  0 / 1          fuse_stub  0: stub kernel + combine, 1: moe_a2a_stub_combine
  *   fuse_route    0: moe_a2a_route + dispatch, 1: moe_a2a_route_dispatch when moe_a2a_fused_ok,
- *                 2: moe_a2a_route_dispatch whenever R fits
+ *                 2: moe_a2a_route_dispatch at any size
  *   expert_y      [R,H] (padded layout: [E*max_recv,H]) of out_type, unused (may be NULL) when fuse_stub
  *   max_recv      0 compact layout, > 0 padded layout (see moe_a2a_route)
  */

@@ -1873,6 +1873,7 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
   if (!fused_small_ok(T, K, H) || (force_tile && atoi(force_tile) == 1)) {  // token tiles: any table size
     if (T == 0) return moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets,
                                      slot_of_entry, src_of_slot, meta, status, nullptr, 0, stream_);
+    if (K > kTileMaxOwn) return MOE_A2A_E_SHAPE;
     const int tile = tile_tokens(T, K, H);
     dim3 grid((unsigned)ceil_div(T, tile)), block(kTileThreads);
     if (streams(T, (long long)T * K, H, 2, 2))
@@ -2117,7 +2118,8 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   if (!known_type(in_type) || !known_type(out_type)) return MOE_A2A_E_DTYPE;
   if (fp8_dispatch && !disp_scale) return MOE_A2A_E_NULL;
   if (!fuse_stub && T > 0 && !expert_y) return MOE_A2A_E_NULL;
-  const bool fused = !fp8_dispatch && T > 0 && (fuse_route == 2 || fuse_route == 1) && moe_a2a_fused_ok(T, K, H);
+  const bool fused = !fp8_dispatch && T > 0 &&
+                     (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
   if (fused) {
     if (int rc = moe_a2a_route_dispatch(x, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts, offsets,
                                         slot_of_entry, src_of_slot, meta, status, disp, stream))
