@@ -22,6 +22,10 @@ per (row, 128-column block) ``amax = max|f32(x)|``, ``scale = amax / 448`` in f3
 (``scale = 1`` when ``amax == 0``), ``q = (f32(x) / scale).to(float8_e4m3fn)``.
 PARITY UNPINNED against the reference for that function (nothing to pin against);
 it is pinned against torch's own e4m3fn cast and the stated error bound only.
+
+``expert_gemm`` / ``expert_gemm_fp8`` (a per-expert linear layer in place of the stub) have no
+counterpart in the reference either: PARITY UNPINNED against it; they are an f32 torch matmul per
+segment and serve as the tolerance reference for the HIP grouped GEMM.
 """
 from __future__ import annotations
 
