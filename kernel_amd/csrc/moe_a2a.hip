@@ -1854,7 +1854,10 @@ int moe_a2a_fused_ok(int T, int K, int H) {
   if (fused_small_ok(T, K, H)) return 1;
   // Token tiles pay off while the rows stay cache-resident (measured: 26 against 35 us at 134 MB of
   // rows, 151 against 110 us at 537 MB); the streaming sizes keep separate routing and dispatch.
-  return streams(T, (long long)T * K, H, 2, 2) ? 0 : 1;
+  if (streams(T, (long long)T * K, H, 2, 2)) return 0;
+  // ... and while a tile of at most kTileMaxOwn entries still keeps the table passes of all
+  // workgroups together below the bytes the dispatch writes: (T / tile) * R * 4 <= R * H * 2
+  return (long long)tile_tokens(T, K, H) * H >= 2ll * T ? 1 : 0;
 }
 
 int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,

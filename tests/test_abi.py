@@ -58,6 +58,7 @@ def test_version_strings_and_queries(lib):
     assert lib.moe_a2a_fused_ok(1024, 6, 2048) == 1  # mid-size table: one launch with token tiles
     assert lib.moe_a2a_fused_ok(2048, 4, 2048) == 1
     assert lib.moe_a2a_fused_ok(4096, 8, 7168) == 0  # streaming sizes keep separate routing and dispatch
+    assert lib.moe_a2a_fused_ok(33000, 8, 64) == 0  # short rows, long table: the table passes would outweigh the rows
 
 
 def test_route_rejects_bad_arguments(lib):

@@ -110,6 +110,47 @@ def test_multi_workgroup_routing(gpu_device):
     compare(cfg, world, gpu_device, C.STUB_EXPERT_FRACTION)
 
 
+@pytest.mark.parametrize("name,scale", [("tiny", 1.0), ("dsv3_rank", 1.0), ("skew_world", 1.0), ("prefill_graph", 1 / 16)])
+@pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
+def test_token_tile_kernel_on_every_size(gpu_device, monkeypatch, name, scale, padded):
+    """The one-launch routing + dispatch with a tile of tokens per workgroup, forced for shapes the
+    library would give to the one-token kernel or to separate launches: same bits everywhere."""
+    monkeypatch.setenv("MOE_A2A_ROUTE_TILE", "1")
+    wl = C.generate_workload(name, tokens_scale=scale)
+    cfg = wl.cfg
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    T = x.shape[0]
+    ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fuse_route="always", padded=padded,
+                      max_recv=T if padded else None)
+    lib = ata.lib
+    import ctypes
+    assert lib.moe_a2a_timer_begin(8) == 0
+    d = ata.dispatch(x, idx, rs)
+    torch.cuda.synchronize()
+    ids, us = (ctypes.c_int * 8)(), (ctypes.c_float * 8)()
+    assert lib.moe_a2a_timer_end(ids, us, 8) == 1
+    assert lib.moe_a2a_kernel_name(ids[0]) == b"route_dispatch_tile"
+    o = V.run_world(cfg, wl.world, stub_kind=wl.stub_kind)
+    assert int(d.status.item()) == 0
+    assert_same("counts", d.counts, o["counts"])
+    assert_same("offsets", d.offsets, o["offsets"])
+    soe = o["slot_of_entry"].long()
+    if padded:
+        e = o["meta"][:, 0].long()
+        want_rows = e * T + (torch.arange(soe.numel()) - o["offsets"].long()[e])  # row of compact slot s
+        assert_same("slot_of_entry", d.slot_of_entry, want_rows[soe].to(torch.int32))
+        rows = d.slot_of_entry.long()
+        assert_same("meta", d.meta[rows], o["meta"][soe])
+        assert_same("disp_x", d.disp_x[rows], o["disp_x"][soe])
+    else:
+        assert_same("slot_of_entry", d.slot_of_entry, o["slot_of_entry"])
+        assert_same("src_of_slot", d.src_of_slot, o["src_of_slot"])
+        assert_same("meta", d.meta, o["meta"])
+        assert_same("disp_x", d.disp_x, o["disp_x"])
+    y = ata.combine(None, w, d, ata.expert_stub(d))
+    assert_same("y", y, o["y"])
+
+
 def test_huge_routing_table(gpu_device):
     """R = 264000 routed rows: more tiles than the rank kernel sums by itself, so the
     column-scan kernel runs too."""
