@@ -309,7 +309,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_tiles_kernel(RouteArgs a)
   if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank, rest[e]);
 }
 
-// Routing in three launches for larger tables.
+// Routing in two or three launches for larger tables.
 // step 1: rows per (tile, expert), tile-major so that lane e reads and writes coalesced.
 __global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(RouteArgs a, int32_t* tile_hist) {
   extern __shared__ int smem[];
@@ -397,6 +397,70 @@ __global__ __launch_bounds__(kRouteThreads) void route_rank_kernel(RouteArgs a, 
   }
   __syncthreads();
   if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank, a.pad ? a.offsets[e] : 0);
+}
+
+// steps 2 and 3 in one launch for up to kRouteFoldMaxTiles tiles: every workgroup sums the columns
+// of the raw (tile, expert) counts for itself -- all tiles for the segment starts, the tiles before
+// its own for its base -- instead of waiting for a one-workgroup scan launch.  The matrix is a few
+// tens of KB and stays in L2; floor(1024 / E) threads share a column as in the scan kernel.
+constexpr int kRouteFoldMaxTiles = 256;
+__global__ __launch_bounds__(kRouteThreads) void route_rank_fold_kernel(RouteArgs a, const int32_t* tile_hist,
+                                                                         int ntiles) {
+  extern __shared__ int smem[];
+  int* wcnt = smem;
+  int* starts = wcnt + kRouteWaves * a.E;
+  __shared__ int part_all[kRouteThreads];
+  __shared__ int part_before[kRouteThreads];
+  __shared__ int s_first[MOE_A2A_MAX_EXPERTS];  // first slot of each expert
+  __shared__ int tmp[kRouteWaves + 1];
+  const int tid = threadIdx.x;
+  load_starts(a, starts);
+  const int i = blockIdx.x * kRouteThreads + tid;
+  const bool valid = i < a.R;
+  const int e = load_expert(a, i, valid);
+  const int parts = kRouteThreads / a.E;  // >= 1 because E <= 1024
+  const int p = tid / a.E, col = tid - p * a.E;
+  const bool live = p < parts;
+  const int span = (ntiles + parts - 1) / parts;
+  const int lo = min(p * span, ntiles), hi = live ? min(lo + span, ntiles) : lo;
+  int all = 0, before = 0;
+  for (int b0 = lo; b0 < hi; b0 += 8) {
+    int c[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) c[u] = b0 + u < hi ? tile_hist[(size_t)(b0 + u) * a.E + col] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      all += c[u];
+      before += b0 + u < (int)blockIdx.x ? c[u] : 0;
+    }
+  }
+  part_all[tid] = live ? all : 0;
+  part_before[tid] = live ? before : 0;
+  const int rank = tile_wave_counts(wcnt, a.E, e, valid, a.nbits);  // its barriers publish the partial sums
+  int column = 0, bef = 0;
+  if (tid < a.E)
+    for (int q = 0; q < parts; ++q) {
+      column += part_all[q * a.E + tid];
+      bef += part_before[q * a.E + tid];
+    }
+  int total;
+  const int excl = block_exclusive_scan(tid < a.E ? column : 0, tmp, total);
+  if (tid < a.E) {
+    s_first[tid] = excl;
+    if (blockIdx.x == 0) {
+      a.counts[tid] = column;
+      a.offsets[tid] = excl;
+    }
+    int run = excl + bef;
+    for (int w = 0; w < kRouteWaves; ++w) {
+      int c = wcnt[w * a.E + tid];
+      wcnt[w * a.E + tid] = run;
+      run += c;
+    }
+  }
+  if (blockIdx.x == 0 && tid == 0) a.offsets[a.E] = total;
+  __syncthreads();
+  if (valid) emit_entry(a, starts, i, e, wcnt[(tid / kWave) * a.E + e] + rank, a.pad ? s_first[e] : 0);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1767,6 +1831,11 @@ int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_ran
   set_max_lds(route_hist_kernel, lds_w);
   if (int rc = launch(KID_ROUTE_HIST, route_hist_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w, stream, a, tile))
     return rc;
+  if (ntiles <= kRouteFoldMaxTiles) {  // scan folded into the rank launch
+    set_max_lds(route_rank_fold_kernel, lds_w + lds_starts);
+    return launch(KID_ROUTE_RANK, route_rank_fold_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w + lds_starts,
+                  stream, a, (const int32_t*)tile, ntiles);
+  }
   if (int rc = launch(KID_ROUTE_SCAN, route_scan_kernel, dim3(1), dim3(kRouteThreads), 0, stream, tile, E, ntiles,
                       counts, offsets))
     return rc;
