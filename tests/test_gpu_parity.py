@@ -195,6 +195,50 @@ def test_limits_and_generic_topk(gpu_device, E, K, T, H):
             compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, combine_mode=mode, fuse_route=fuse)
 
 
+def _random_shapes(n, seed):
+    """Seeded sweep of routing shapes around the limits that pick a kernel: entries per thread of the
+    one-token kernel (4..32), its table-read budget, tile sizes of the token-tile kernel, one
+    workgroup vs. several routing tiles, ragged worlds, duplicate-free and duplicated expert ids."""
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+    out = []
+    for _ in range(n):
+        W = pick([1, 2, 4, 8])
+        E = W * pick([1, 2, 3, 8, 16, 32])
+        K = pick([1, 2, 3, 4, 6, 8, 12])
+        H = 8 * pick([1, 3, 8, 32, 96, 129, 256, 512])
+        T = pick([1, 2, 5, 31, 64, 129, 300, 777, 1500, 2500])
+        out.append((W, E, K, H, T, bool(pick([0, 0, 1])), int(torch.randint(0, 1 << 30, (1,), generator=g))))
+    return out
+
+
+@pytest.mark.parametrize("W,E,K,H,T,dup,seed", _random_shapes(24, 2024))
+def test_random_shapes_all_routing_kernels(gpu_device, monkeypatch, W, E, K, H, T, dup, seed):
+    """Every routing implementation (one-token, token-tile, separate launches) on the same random
+    world, compact and through the library's own choice: all bit-identical to the oracle."""
+    g = torch.Generator().manual_seed(seed)
+    K = min(K, E) if not dup else K
+    cfg = C.MoEConfig(E, K, H, T + 1, torch.bfloat16, torch.bfloat16)
+    cuts = sorted(int(v) for v in torch.randint(0, T + 1, (W - 1,), generator=g)) if W > 1 else []
+    cuts = [0] + cuts + [T]
+    world = []
+    for r in range(W):
+        n = cuts[r + 1] - cuts[r]
+        if dup:
+            idx = torch.randint(0, E, (n, K), generator=g).to(torch.int32)
+        else:
+            idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(n)]).to(torch.int32) if n else \
+                torch.empty(0, K, dtype=torch.int32)
+        world.append(C.RankData(n, idx, torch.rand(n, K, generator=g), torch.randn(n, H, generator=g).to(torch.bfloat16)))
+    monkeypatch.delenv("MOE_A2A_ROUTE_TILE", raising=False)
+    compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=True)       # the library's choice
+    compare(cfg, world, gpu_device, C.STUB_EXPERT_FRACTION, fuse_route=False)  # separate launches
+    monkeypatch.setenv("MOE_A2A_ROUTE_TILE", "1")
+    compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route="always")   # token tiles
+    monkeypatch.setenv("MOE_A2A_ROUTE_TILE", "0")
+    compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route="always")   # one-token kernel when it applies
+
+
 @pytest.mark.parametrize("name", ["tiny", "dsv3_rank", "skew_world"])
 def test_forward_single_call_equals_separate_calls(gpu_device, name):
     wl = C.generate_workload(name)
