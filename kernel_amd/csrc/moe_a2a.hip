@@ -35,7 +35,6 @@ constexpr int kRouteTilesMaxRows = 16 * kRouteThreads;  // one-launch routing up
 constexpr int kRowMaxThreads = 512;
 constexpr int kFusedIdBits = 13;
 constexpr int kFusedMaxRows = 1 << kFusedIdBits;  // route_dispatch packs (expert, entry id) into one key
-constexpr int kFusedMaxEntriesPerThread = 32;
 constexpr int kFusedMaxThreads = 1024;
 #ifndef MOE_A2A_FUSED_TABLE_READS
 #define MOE_A2A_FUSED_TABLE_READS (1ll << 20)
