@@ -59,6 +59,8 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--cold", action="store_true", help="add a leg with caches flushed before every step")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
+    p.add_argument("--fp8-weights", action="store_true",
+                   help="with --expert-gemm: weights as e4m3fn bytes with one f32 scale per 128 x 128 block")
     p.add_argument("--expert-gemm", type=int, default=0, metavar="N",
                    help="measure the grouped expert GEMM (N output columns per expert) on the workload's "
                         "dispatched rows instead of the dispatch/combine path")
@@ -322,6 +324,12 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
     ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fp8_dispatch=fp8)
     gen = torch.Generator(device="cpu").manual_seed(1234)
     weights = (torch.randn(E, N, H, generator=gen) / H ** 0.5).to(cfg.in_dtype).to(dev)
+    w_scale = None
+    if args.fp8_weights:  # block quantisation of the synthetic weights (input preparation, not timed)
+        wf = weights.float().view(E, N // 128, 128, H // 128, 128)
+        amax = wf.abs().amax(dim=(2, 4))
+        w_scale = torch.where(amax == 0, torch.ones_like(amax), amax / 448.0).contiguous()
+        weights = (wf / w_scale[:, :, None, :, None]).to(torch.float8_e4m3fn).view(E, N, H).contiguous()
     main = torch.cuda.Stream()
     main.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(main):
@@ -329,13 +337,13 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
         R = d.num_rows
         y = torch.empty(R, N, dtype=cfg.in_dtype, device=dev)
         for _ in range(args.warmup):
-            ata.expert_gemm(d, weights, out=y)
+            ata.expert_gemm(d, weights, out=y, w_scale=w_scale)
         main.synchronize()
-        per = kernel_times(lib, lambda n: [ata.expert_gemm(d, weights, out=y) for _ in range(n)], args.steps, torch)
+        per = kernel_times(lib, lambda n: [ata.expert_gemm(d, weights, out=y, w_scale=w_scale) for _ in range(n)], args.steps, torch)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(main)
         for _ in range(args.steps):
-            ata.expert_gemm(d, weights, out=y)
+            ata.expert_gemm(d, weights, out=y, w_scale=w_scale)
         e1.record(main)
         main.synchronize()
     ms_step = e0.elapsed_time(e1) / args.steps
@@ -348,13 +356,14 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
                scaling="weak", vs_baseline=None, dtype="bf16" if cfg.in_dtype == torch.bfloat16 else "f16",
                data="synthetic",
                config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N, kernel=kernel,
-                           rows_dtype="fp8 e4m3fn + f32 scale per 128 columns" if fp8 else "16-bit"),
+                           rows_dtype="fp8 e4m3fn + f32 scale per 128 columns" if fp8 else "16-bit",
+                           weights_dtype="fp8 e4m3fn + f32 scale per 128 x 128 block" if args.fp8_weights else "16-bit"),
                kernels_us=summarise(per),
                )
     # which roof: the operands must cross HBM once (rows, the weights of every expert that has rows,
     # the output); if that takes longer at 8 TB/s than the flops at the MFMA peak, the launch is HBM-bound
     live = int((d.counts > 0).sum())
-    gemm_bytes = R * H * (1 + 4 / 128 if fp8 else 2) + live * N * H * 2 + R * N * 2
+    gemm_bytes = R * H * (1 + 4 / 128 if fp8 else 2) + live * N * H * (1 if args.fp8_weights else 2) + R * N * 2
     if gemm_bytes / (HBM_PEAK_GBPS * 1e3) > flops / (MFMA_PEAK_TFLOPS * 1e6):
         gbps = gemm_bytes / t_us / 1e3
         out["roofline"] = dict(bound="hbm", achieved=round(gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
@@ -373,7 +382,10 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
             lo, hi = int(off[e]), int(off[e + 1])
             if hi > lo:
                 seg = torch.tensor([0, hi - lo], dtype=torch.int32)
-                if fp8:
+                if args.fp8_weights:
+                    ref = O.expert_gemm_q8(dx[lo:hi], dsc[lo:hi] if fp8 else None, wc[e:e + 1].view(torch.uint8),
+                                           w_scale[e:e + 1].cpu(), seg, cfg.in_dtype)
+                elif fp8:
                     ref = O.expert_gemm_fp8(dx[lo:hi], dsc[lo:hi], seg, wc[e:e + 1], cfg.in_dtype)
                 else:
                     ref = O.expert_gemm(dx[lo:hi], seg, wc[e:e + 1], cfg.in_dtype)

@@ -208,6 +208,19 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
                             moe_a2a_stream_t stream);
 
 /*
+ * The same product with quantised weights in the block format of DeepSeek-V3 checkpoints:
+ * w_q[E, N, Kd] e4m3fn bytes with w_scale[E, N/128, Kd/128] f32 (one scale per 128 x 128 block).
+ * x is 16-bit (x_scale == NULL) or the e4m3fn rows + x_scale[rows, Kd/128] of moe_a2a_dispatch_fp8.
+ * y = sum over K blocks of scale_b * (x . q_b): the weight bytes enter the matrix cores exactly, each
+ * 128-wide block is summed in f32 and scaled in f32 (fp8 rows of x are dequantised and rounded once
+ * to elem_type first); y[rows, N] of elem_type.  Kd % 128 == 0, N % 128 == 0.  The weights cross memory
+ * as one byte per element, which is what bounds a decode step.  No counterpart in the reference.
+ */
+int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
+                           const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
+                           moe_a2a_stream_t stream);
+
+/*
  * Launch timer (opt-in, process-wide, single caller thread).  Between begin and end every
  * kernel the library launches carries a pair of HIP events bound to that dispatch, so the
  * reported time is the kernel's own begin-to-end duration on the GPU.

@@ -229,7 +229,8 @@ class HipAllToAll:
                                          _ptr(y), R, H, _stream()), "moe_a2a_stub")
         return y
 
-    def expert_gemm(self, d: Dispatched, weights: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def expert_gemm(self, d: Dispatched, weights: torch.Tensor, out: Optional[torch.Tensor] = None,
+                    w_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Real expert compute in place of the stub: ``y[rows of e] = disp_x[rows of e] @ weights[e].T``
         for every expert, on the matrix cores (f32 accumulation, one rounding to ``out_dtype``).
 
@@ -237,31 +238,42 @@ class HipAllToAll:
         dispatched buffer (rows that hold no entry are not written).  ``N == H`` feeds ``combine``.
         16-bit dispatched rows must have the weights' type; fp8 dispatched rows (``d.disp_scale``
         set) are dequantised inside the kernel, each element rounded once to the weights' type.
+
+        Block-quantised weights: ``weights`` as e4m3fn bits (``uint8`` or ``float8_e4m3fn``) with
+        ``w_scale[E, N/128, H/128]`` f32, the format of DeepSeek-V3 checkpoints; ``N % 128 == 0``.
         """
         cfg = self.cfg
         _require_gpu(weights, "weights")
         rows, H = d.disp_x.shape
         E = cfg.num_experts
-        if weights.dim() != 3 or weights.shape[0] != E or weights.shape[2] != H or weights.dtype != cfg.out_dtype \
+        quant = w_scale is not None
+        want_w = (torch.uint8, torch.float8_e4m3fn) if quant else (cfg.out_dtype,)
+        if weights.dim() != 3 or weights.shape[0] != E or weights.shape[2] != H or weights.dtype not in want_w \
                 or not weights.is_contiguous():
-            raise ValueError("weights must be out_dtype[E, N, H], contiguous")
+            raise ValueError("weights must be out_dtype[E, N, H] (or e4m3fn bits with w_scale), contiguous")
         fp8 = d.disp_scale is not None
         if not fp8 and cfg.out_dtype != d.disp_x.dtype:
             raise ValueError("expert_gemm keeps the element type of 16-bit dispatched rows")
         N = weights.shape[1]
+        if quant:
+            _require_gpu(w_scale, "w_scale")
+            if H % 128 or N % 128 or tuple(w_scale.shape) != (E, N // 128, H // 128) or w_scale.dtype != torch.float32 \
+                    or not w_scale.is_contiguous():
+                raise ValueError("w_scale must be float32[E, N/128, H/128], contiguous, with N and H multiples of 128")
         if out is None:
             out = torch.empty(rows, N, dtype=cfg.out_dtype, device=weights.device)
         elif tuple(out.shape) != (rows, N) or out.dtype != cfg.out_dtype or not out.is_contiguous():
             raise ValueError("out must be out_dtype[rows, N], contiguous")
-        if fp8:
-            _lib.check(self.lib.moe_a2a_expert_gemm_fp8(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(weights),
-                                                        _ptr(d.offsets), _ptr(out), d.num_rows, E, H, N, d.max_recv,
-                                                        _elem(cfg.out_dtype), _stream()),
+        common = (_ptr(d.offsets), _ptr(out), d.num_rows, E, H, N, d.max_recv, _elem(cfg.out_dtype), _stream())
+        if quant:
+            _lib.check(self.lib.moe_a2a_expert_gemm_q8(_ptr(d.disp_x), _ptr(d.disp_scale) if fp8 else None,
+                                                       _ptr(weights), _ptr(w_scale), *common),
+                       "moe_a2a_expert_gemm_q8")
+        elif fp8:
+            _lib.check(self.lib.moe_a2a_expert_gemm_fp8(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(weights), *common),
                        "moe_a2a_expert_gemm_fp8")
         else:
-            _lib.check(self.lib.moe_a2a_expert_gemm(_ptr(d.disp_x), _ptr(weights), _ptr(d.offsets), _ptr(out),
-                                                    d.num_rows, E, H, N, d.max_recv, _elem(cfg.out_dtype), _stream()),
-                       "moe_a2a_expert_gemm")
+            _lib.check(self.lib.moe_a2a_expert_gemm(_ptr(d.disp_x), _ptr(weights), *common), "moe_a2a_expert_gemm")
         return out
 
     # ---- combine ---------------------------------------------------------------------

@@ -1463,6 +1463,182 @@ __device__ __forceinline__ void wide_decode_fp8(const u32x4_t& q, float scale, u
   hi = u32x4_t{o[4], o[5], o[6], o[7]};
 }
 
+// 16 fp8 (e4m3fn) values -> two vectors of 8 values of E, exactly (every e4m3fn value is a bf16 and
+// an f16 value)
+template <class E>
+__device__ __forceinline__ void exact_fp8_to_16(const u32x4_t& q, u32x4_t& lo, u32x4_t& hi) {
+  uint32_t o[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float f[4];
+    fp8x4_to_f32(q[j], f);
+    o[2 * j] = E::pack(f[0], f[1]);
+    o[2 * j + 1] = E::pack(f[2], f[3]);
+  }
+  lo = u32x4_t{o[0], o[1], o[2], o[3]};
+  hi = u32x4_t{o[4], o[5], o[6], o[7]};
+}
+
+// The weight-streaming kernel for quantised operands (the block format of DeepSeek-V3 checkpoints):
+// weights as e4m3fn bytes with one f32 scale per 128 x 128 block, activations either 16-bit or the
+// e4m3fn rows + per-(row, 128 columns) scales that dispatch_fp8 writes (AFP8).  Tile 32 x 128, K
+// slabs of 128, so a workgroup meets exactly one weight scale per slab: the weight bytes go into
+// LDS as exact 16-bit values, each slab is summed on the matrix cores into a partial accumulator,
+// and the partial is folded into the result with one fma per element, acc += scale * partial --
+// y = sum over K blocks of scale_b * (x . q_b), the scale applied in f32 after the block sum.
+// Activation rows are dequantised on their way into LDS, E(f32(q) * scale) (they are a thousandth
+// of the traffic here).  The weights cross HBM as one byte per element, which is what bounds a
+// decode step; four slabs are in flight per workgroup in four register sets.
+template <class E, bool AFP8>
+__global__ __launch_bounds__(kSkinnyThreads, 3) void expert_gemm_skinny_q_kernel(
+    const uint4* __restrict__ x, const float* __restrict__ x_scale, const uint4* __restrict__ w,
+    const float* __restrict__ w_scale, const int32_t* __restrict__ offsets, uint16_t* __restrict__ y,
+    int num_experts, int Kd, int N, int max_recv, int ntile_n) {
+  constexpr int TM = kSkinnyM, TN = 128, BK = 128, LD = BK + 8, NT = kSkinnyThreads;  // Kd % 128 == 0, N % 128 == 0
+  __shared__ __attribute__((aligned(16))) uint16_t s_ab[(TM + TN) * LD];
+  uint16_t* s_a = s_ab;
+  uint16_t* s_b = s_ab + TM * LD;
+  __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
+  __shared__ int s_tmp[NT / kWave + 1];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int tile_n = blockIdx.x % ntile_n;
+  const int tile_m_global = blockIdx.x / ntile_n;
+  {
+    const int span = (num_experts + NT - 1) / NT;
+    const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    int total;
+    int run = block_exclusive_scan(sum, s_tmp, total);
+    for (int e = lo; e < hi; ++e) {
+      s_pref[e] = run;
+      run += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    }
+    if (tid == 0) s_pref[num_experts] = total;
+    __syncthreads();
+    if (tile_m_global >= total) return;
+  }
+  int e_lo = 0, e_hi = num_experts;
+  while (e_hi - e_lo > 1) {
+    int mid = (e_lo + e_hi) >> 1;
+    if (s_pref[mid] <= tile_m_global) e_lo = mid; else e_hi = mid;
+  }
+  const int e = __builtin_amdgcn_readfirstlane(e_lo);  // the same in every lane: scales load as scalars
+  const int count = offsets[e + 1] - offsets[e];
+  const int m0 = (tile_m_global - s_pref[e]) * TM;
+  const size_t row0 = (size_t)(max_recv > 0 ? e * max_recv : offsets[e]) + m0;
+  const int rows = min(TM, count - m0);
+  const int n0 = tile_n * TN;
+  const int kblocks = Kd / 128;
+  // vectors of 16 bytes: 8 elements of a 16-bit operand, 16 of an fp8 one
+  constexpr int AV = AFP8 ? BK / 16 : BK / 8, BV = BK / 16;  // per row and slab
+  constexpr int NA = TM * AV / NT, NB = TN * BV / NT;         // per thread: 1 or 2, and 4
+  static_assert(NA >= 1, "a slab of A holds at least one vector per thread");
+  const int a_row_vecs = AFP8 ? Kd / 16 : Kd / 8, b_row_vecs = Kd / 16;
+  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * a_row_vecs;
+  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * b_row_vecs;
+  const float* xs = AFP8 ? x_scale + row0 * kblocks : nullptr;
+  const float* ws = w_scale + ((size_t)e * (N / 128) + tile_n) * kblocks;
+  int offa[NA], offs[NA], sta[NA], offb[NB], stb[NB];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int v = tid + i * NT, r = v / AV, c = v % AV;
+    offa[i] = min(r, rows - 1) * a_row_vecs + c;
+    offs[i] = min(r, rows - 1) * kblocks;
+    sta[i] = r * LD + c * (AFP8 ? 16 : 8);
+  }
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int v = tid + i * NT, r = v / BV, c = v % BV;
+    offb[i] = r * b_row_vecs + c;  // N % 128 == 0: every column of the tile exists
+    stb[i] = r * LD + c * 16;
+  }
+  struct Slab {
+    u32x4_t a[NA], b[NB];
+    float as[NA];
+    float bs;
+  };
+  Slab s0, s1, s2, s3;
+#define SKQ_FETCH(S, K0)                                                                              \
+  {                                                                                                   \
+    const int k_ = min((K0), Kd - BK); /* past the end: the last slab again */                        \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i) {                                                  \
+      S.a[i] = xa[offa[i] + (k_ >> (AFP8 ? 4 : 3))];                                                  \
+      S.as[i] = AFP8 ? xs[offs[i] + (k_ >> 7)] : 1.f;                                                 \
+    }                                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) S.b[i] = __builtin_nontemporal_load(wb + offb[i] + (k_ >> 4)); \
+    S.bs = ws[k_ >> 7];                                                                               \
+  }
+#define SKQ_STASH(S)                                                                                  \
+  {                                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i) {                                                  \
+      if (AFP8) {                                                                                     \
+        u32x4_t lo_, hi_;                                                                             \
+        wide_decode_fp8<E>(S.a[i], S.as[i], lo_, hi_);                                                \
+        *reinterpret_cast<u32x4_t*>(&s_a[sta[i]]) = lo_;                                              \
+        *reinterpret_cast<u32x4_t*>(&s_a[sta[i] + 8]) = hi_;                                          \
+      } else {                                                                                        \
+        *reinterpret_cast<u32x4_t*>(&s_a[sta[i]]) = S.a[i];                                           \
+      }                                                                                               \
+    }                                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) {                                                  \
+      u32x4_t lo_, hi_;                                                                               \
+      exact_fp8_to_16<E>(S.b[i], lo_, hi_);                                                           \
+      *reinterpret_cast<u32x4_t*>(&s_b[stb[i]]) = lo_;                                                \
+      *reinterpret_cast<u32x4_t*>(&s_b[stb[i] + 8]) = hi_;                                            \
+    }                                                                                                 \
+  }
+  f32x16_t acc;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) acc[q] = 0.f;
+  const int wn = wave * 32;
+  const int fr_a = (lane & 31) * LD + (lane >> 5) * 8;
+  const int fr_b = (wn + (lane & 31)) * LD + (lane >> 5) * 8;
+#define SKQ_SLAB(SCALE)                                                                               \
+  {                                                                                                   \
+    f32x16_t part;                                                                                    \
+    _Pragma("unroll") for (int q = 0; q < 16; ++q) part[q] = 0.f;                                     \
+    _Pragma("unroll") for (int kk = 0; kk < BK; kk += 16) {                                           \
+      const u32x4_t fa = *reinterpret_cast<const u32x4_t*>(&s_a[fr_a + kk]);                          \
+      const u32x4_t fb = *reinterpret_cast<const u32x4_t*>(&s_b[fr_b + kk]);                          \
+      part = mfma_32x32x16_v<E>(fa, fb, part);                                                        \
+    }                                                                                                 \
+    _Pragma("unroll") for (int q = 0; q < 16; ++q) acc[q] = __builtin_fmaf(part[q], (SCALE), acc[q]); \
+  }
+#define SKQ_STEP(S, KNEXT)                                                                            \
+  {                                                                                                   \
+    SKQ_STASH(S);                                                                                     \
+    const float scale_ = S.bs;                                                                        \
+    __syncthreads();                                                                                  \
+    SKQ_FETCH(S, (KNEXT));                                                                            \
+    SKQ_SLAB(scale_);                                                                                 \
+    __syncthreads();                                                                                  \
+  }
+  SKQ_FETCH(s0, 0);
+  SKQ_FETCH(s1, BK);
+  SKQ_FETCH(s2, 2 * BK);
+  SKQ_FETCH(s3, 3 * BK);
+  for (int k0 = 0; k0 < Kd; k0 += 4 * BK) {
+    SKQ_STEP(s0, k0 + 4 * BK);
+    if (k0 + BK >= Kd) break;
+    SKQ_STEP(s1, k0 + 5 * BK);
+    if (k0 + 2 * BK >= Kd) break;
+    SKQ_STEP(s2, k0 + 6 * BK);
+    if (k0 + 3 * BK >= Kd) break;
+    SKQ_STEP(s3, k0 + 7 * BK);
+  }
+#undef SKQ_FETCH
+#undef SKQ_STASH
+#undef SKQ_SLAB
+#undef SKQ_STEP
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int r = (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
+    const int c = wn + (lane & 31);
+    if (r < rows) y[(row0 + r) * (size_t)N + n0 + c] = (uint16_t)(E::pack(acc[q], 0.f) & 0xffffu);
+  }
+}
+
 // Main loop and epilogue of one wide tile.  Each wave owns WMI x WNJ accumulator blocks of 32 x 32
 // at (wm, wn); AROWS rows of the A operand are staged per slab (256, or 128 when the tile holds
 // no more rows than that), always 256 rows of B.
@@ -2306,6 +2482,34 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
   if (!x_q || !x_scale || !weights || !offsets || !y) return MOE_A2A_E_NULL;
   if (!aligned16(x_q) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
   return launch_gemm_wide(x_q, x_scale, weights, offsets, y, R, E, Kd, N, max_recv, elem_type, (hipStream_t)stream_);
+}
+
+int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
+                           const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
+                           moe_a2a_stream_t stream_) {
+  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
+  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 ||
+      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0)
+    return MOE_A2A_E_SHAPE;
+  if (R == 0) return 0;
+  if (!x || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
+  if (!aligned16(x) || !aligned16(w_q) || !aligned16(y)) return MOE_A2A_E_ALIGN;
+  hipStream_t stream = (hipStream_t)stream_;
+  const int ntile_n = N / 128;
+  const long long mtiles = (long long)R / kSkinnyM + E;
+  if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
+  dim3 grid((unsigned)(mtiles * ntile_n)), block(kSkinnyThreads);
+#define CALL_SKQ(ET, AF)                                                                                        \
+  return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_skinny_q_kernel<ET, AF>, grid, block, 0, stream,       \
+                (const uint4*)x, x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, \
+                ntile_n)
+  if (elem_type == MOE_A2A_BF16) {
+    if (x_scale) CALL_SKQ(Bf16, true);
+    CALL_SKQ(Bf16, false);
+  }
+  if (x_scale) CALL_SKQ(F16, true);
+  CALL_SKQ(F16, false);
+#undef CALL_SKQ
 }
 
 int moe_a2a_timer_begin(int capacity) {

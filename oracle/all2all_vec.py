@@ -156,6 +156,44 @@ def expert_gemm_fp8(q_bits: torch.Tensor, scale: torch.Tensor, offsets: torch.Te
     return expert_gemm(dequantize_fp8(q_bits, scale).to(weights.dtype), offsets, weights, out_dtype)
 
 
+def quantize_weights_fp8(weights: torch.Tensor):
+    """Expert weights ``[E, N, Kd]`` -> e4m3fn bits and one f32 scale per 128 x 128 block
+    (``scale = amax / 448``, 1 for an all-zero block): the block format of DeepSeek-V3 checkpoints.
+    Test-side helper: the library only consumes weights in this format."""
+    E, N, Kd = weights.shape
+    assert N % FP8_BLOCK == 0 and Kd % FP8_BLOCK == 0
+    wf = weights.to(torch.float32).view(E, N // FP8_BLOCK, FP8_BLOCK, Kd // FP8_BLOCK, FP8_BLOCK)
+    amax = wf.abs().amax(dim=(2, 4))
+    scale = torch.where(amax == 0, torch.ones_like(amax), amax / FP8_MAX)
+    q = (wf / scale[:, :, None, :, None]).to(torch.float8_e4m3fn)
+    return q.view(E, N, Kd).view(torch.uint8), scale
+
+
+def dequantize_weights_fp8(q_bits: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    E, N, Kd = q_bits.shape
+    qf = q_bits.view(torch.float8_e4m3fn).to(torch.float32).view(E, N // FP8_BLOCK, FP8_BLOCK, Kd // FP8_BLOCK, FP8_BLOCK)
+    return (qf * scale[:, :, None, :, None]).view(E, N, Kd)
+
+
+def expert_gemm_q8(disp_x: torch.Tensor, x_scale, w_bits: torch.Tensor, w_scale: torch.Tensor,
+                   offsets: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """The expert layer with block-quantised weights: ``y = sum over K blocks of scale_b * (x . q_b)``,
+    i.e. the weights enter exactly (``f32(q) * scale`` in f32) and everything is summed in f32, one
+    rounding to ``out_dtype`` at the end.  fp8 rows (``x_scale`` given) are dequantised and rounded
+    once to ``out_dtype`` first, as in ``expert_gemm_fp8``.  No counterpart in the reference:
+    PARITY UNPINNED against it."""
+    w = dequantize_weights_fp8(w_bits, w_scale)  # f32
+    x = dequantize_fp8(disp_x, x_scale).to(out_dtype) if x_scale is not None else disp_x
+    R = x.shape[0]
+    E, N, _ = w.shape
+    y = torch.zeros(R, N, dtype=out_dtype)
+    off = offsets.tolist()
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            y[off[e]:off[e + 1]] = (x[off[e]:off[e + 1]].float() @ w[e].t()).to(out_dtype)
+    return y
+
+
 def combine_strict(expert_y: torch.Tensor, weights: torch.Tensor, slot_of_entry: torch.Tensor,
                    out_dtype: torch.dtype) -> torch.Tensor:
     """Reference-order weighted sum with a rounding to ``out_dtype`` after every add."""

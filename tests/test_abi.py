@@ -127,6 +127,15 @@ def test_expert_gemm_rejects_bad_arguments(lib):
         assert f(w=None) == E_NULL
         assert f(off=None) == E_NULL
         assert f(y=A + 8) == E_ALIGN
+    def gemmq(x=A, xs=None, w=A, ws=A, off=A, y=A, R=64, E=8, Kd=128, N=128, max_recv=0, elem=_lib.BF16):
+        return lib.moe_a2a_expert_gemm_q8(x, xs, w, ws, off, y, R, E, Kd, N, max_recv, elem, None)
+
+    assert gemmq(elem=5) == E_DTYPE
+    assert gemmq(N=64) == E_SHAPE   # one weight scale per 128 x 128 block
+    assert gemmq(Kd=192) == E_SHAPE
+    assert gemmq(ws=None) == E_NULL
+    assert gemmq(R=0) == 0
+    assert gemmq(y=A + 4) == E_ALIGN
     assert gemm(Kd=72) == E_SHAPE    # hidden size in slabs of 64
     assert gemm8(Kd=192) == E_SHAPE  # fp8 rows carry one scale per 128 columns
     assert gemm8(sc=None) == E_NULL

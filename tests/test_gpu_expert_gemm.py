@@ -161,6 +161,32 @@ def test_decode_shape_takes_the_skinny_kernel(gpu_device, monkeypatch):
     close(y, V.expert_gemm(o["disp_x"], o["offsets"], weights, torch.bfloat16))
 
 
+@pytest.mark.parametrize("E,K,T,H,N,W,zipf", [
+    (8, 2, 40, 128, 128, 1, False),      # one block each way
+    (64, 4, 128, 512, 384, 8, False),    # decode-like: 8 rows per expert
+    (16, 4, 300, 384, 256, 4, True),     # skewed: empty experts and long segments
+    (8, 2, 1200, 256, 256, 2, False),    # 300 rows per expert
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("fp8_rows", [False, True], ids=["rows16", "rows8"])
+@pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
+def test_expert_gemm_block_quantised_weights(gpu_device, E, K, T, H, N, W, zipf, dtype, fp8_rows, padded):
+    """Weights as e4m3fn bytes with one scale per 128 x 128 block, rows 16-bit or from the fp8
+    dispatch, against an f32 matmul of the dequantised operands (each rounded once to the 16-bit
+    type, as the kernel does)."""
+    cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=5 * E + T, zipf=zipf)
+    wq, ws = V.quantize_weights_fp8(weights)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, fp8_dispatch=fp8_rows, padded=padded, max_recv=T if padded else None)
+    d = ata.dispatch(x, idx, rs)
+    y = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device))
+    torch.cuda.synchronize()
+    o = V.run_world(cfg, world, fp8=fp8_rows)
+    want = V.expert_gemm_q8(o["disp_x"], o["disp_scale"] if fp8_rows else None, wq, ws, o["offsets"], dtype)
+    rows = d.slot_of_entry.long() if padded else o["slot_of_entry"].long().to(gpu_device)
+    close(y[rows], want[o["slot_of_entry"].long()])
+
+
 def test_dispatch_gemm_combine_end_to_end(gpu_device):
     """dispatch -> expert GEMM (H -> H) -> combine against the same chain on the CPU."""
     cfg, world, weights = make(32, 4, 512, 256, 256, 8, torch.bfloat16, seed=3)
