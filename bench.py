@@ -390,8 +390,9 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
                 else:
                     ref = O.expert_gemm(dx[lo:hi], seg, wc[e:e + 1], cfg.in_dtype)
                 want, got = ref.float(), yg[lo:hi].float()
-                # summation order differs from the CPU's: 1 % of the value + 1 % of the segment's rms
-                tol = 1e-2 * want.abs() + 1e-2 * want.pow(2).mean().sqrt()
+                # summation order (and, for quantised weights on long segments, one rounding of the
+                # dequantised weight) differs from the CPU's: 1 % of the value + 1 % of the row's rms
+                tol = 1e-2 * want.abs() + 1e-2 * want.pow(2).mean(dim=1, keepdim=True).sqrt()
                 worst = max(worst, float(((got - want).abs() / tol).max()))
                 rows_done += hi - lo
             done += 1

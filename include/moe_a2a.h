@@ -210,11 +210,18 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
 /*
  * The same product with quantised weights in the block format of DeepSeek-V3 checkpoints:
  * w_q[E, N, Kd] e4m3fn bytes with w_scale[E, N/128, Kd/128] f32 (one scale per 128 x 128 block).
- * x is 16-bit (x_scale == NULL) or the e4m3fn rows + x_scale[rows, Kd/128] of moe_a2a_dispatch_fp8.
- * y = sum over K blocks of scale_b * (x . q_b): the weight bytes enter the matrix cores exactly, each
- * 128-wide block is summed in f32 and scaled in f32 (fp8 rows of x are dequantised and rounded once
- * to elem_type first); y[rows, N] of elem_type.  Kd % 128 == 0, N % 128 == 0.  The weights cross memory
- * as one byte per element, which is what bounds a decode step.  No counterpart in the reference.
+ * x is 16-bit (x_scale == NULL) or the e4m3fn rows + x_scale[rows, Kd/128] of moe_a2a_dispatch_fp8
+ * (dequantised and rounded once to elem_type inside the kernel); y[rows, N] of elem_type.
+ * Kd % 128 == 0, N % 128 == 0.  Two kernels, chosen by the mean segment length:
+ *   R <= 32 * E (a decode step, bound by the weight bytes, which cross memory once at one byte per
+ *     element): 32 x 128 tiles; the weight bytes enter the matrix cores exactly, each 128-wide K
+ *     block is summed in f32 and scaled in f32: y = sum over K blocks of scale_b * (x . q_b).
+ *   longer segments (and N >= 256): the 256 x 256 kernel; a weight enters the matrix cores as
+ *     elem(f32(q) * scale), i.e. dequantised and rounded once to elem_type on its way into LDS --
+ *     the result of dequantising the weights to 16 bits and calling moe_a2a_expert_gemm, without
+ *     the 16-bit copy in memory.
+ * The two differ by that one rounding of a weight (2^-9 relative for bf16); MOE_A2A_GEMM_TILE=32 or
+ * 256 forces one.  No counterpart in the reference.
  */
 int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,

@@ -1642,23 +1642,26 @@ __global__ __launch_bounds__(kSkinnyThreads, 3) void expert_gemm_skinny_q_kernel
 // Main loop and epilogue of one wide tile.  Each wave owns WMI x WNJ accumulator blocks of 32 x 32
 // at (wm, wn); AROWS rows of the A operand are staged per slab (256, or 128 when the tile holds
 // no more rows than that), always 256 rows of B.
-template <class E, int WMI, int WNJ, int AROWS, bool AFP8>
+template <class E, int WMI, int WNJ, int AROWS, bool AFP8, bool BFP8>
 __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const float* __restrict__ xs,
-                                          const u32x4_t* __restrict__ wb, uint16_t* __restrict__ y_tile,
-                                          uint16_t* s_wide, int rows, int ncols, int Kd, int N, int wm, int wn) {
+                                          const u32x4_t* __restrict__ wb, const float* __restrict__ wsc,
+                                          uint16_t* __restrict__ y_tile, uint16_t* s_wide, int rows, int ncols,
+                                          int Kd, int N, int wm, int wn) {
   constexpr int TM = kWideM, TN = kWideN, BK = kWideK, LD = kWideLd, NT = kWideThreads;
   const int tid = threadIdx.x, lane = tid & (kWave - 1);
   const int kvec = Kd / 8;
   // A slab is AROWS (A) + 256 (B) rows of 64 elements.  Rows past the segment and columns past N
   // read the last valid row instead of zeros: they only feed accumulators that are never stored,
-  // and the loads stay unconditional.  16-bit A: 8 vectors of 8 elements per row.  fp8 A (AFP8): 4
-  // vectors of 16 elements per row plus the row's f32 scale of that 128-column block; a vector is
-  // turned into two 16-bit vectors, E(f32(q) * scale), on its way into LDS, so the LDS image, the
-  // number of LDS stores and the number of global loads per thread are those of the 16-bit case.
-  constexpr int VPR = BK / 8, NB = TN * VPR / NT;
-  constexpr int AVPR = AFP8 ? BK / 16 : VPR;      // global A vectors per row and slab
-  constexpr int NA = AROWS * AVPR / NT;            // ... per thread
-  constexpr int NS = AFP8 ? NA : 0;                // scales per thread
+  // and the loads stay unconditional.  A 16-bit operand: 8 vectors of 8 elements per row.  An fp8
+  // operand: 4 vectors of 16 elements per row plus a scale -- for A (AFP8) the row's f32 scale of
+  // that 128-column block, for B (BFP8) the scale of the 128 x 128 weight block (two column blocks
+  // per tile: wsc[0..] and wsc[Kd/128..]); a vector is turned into two 16-bit vectors,
+  // E(f32(q) * scale), on its way into LDS, so the LDS image and the number of LDS stores per
+  // thread are those of the 16-bit case.
+  constexpr int VPR = BK / 8;
+  constexpr int AVPR = AFP8 ? BK / 16 : VPR, BVPR = BFP8 ? BK / 16 : VPR;  // global vectors per row and slab
+  constexpr int NA = AROWS * AVPR / NT, NB = TN * BVPR / NT;               // ... per thread
+  constexpr int NS = AFP8 ? NA : 0;                                         // A scales per thread
   int offa[NA], offs[NS > 0 ? NS : 1], offb[NB];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
@@ -1670,24 +1673,29 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const int v = tid + i * NT;
-    offb[i] = min(v / VPR, ncols - 1) * kvec + v % VPR;
+    offb[i] = min(v / BVPR, ncols - 1) * (BFP8 ? Kd / 16 : kvec) + v % BVPR;
   }
   // native vectors, not uint4: the struct type keeps the staging arrays in scratch memory
   u32x4_t ra[NA], rb[NB];
   float rs[NS > 0 ? NS : 1];
-  const int st_off = (tid / VPR) * LD + (tid % VPR) * 8;
-  const int st_off_a = AFP8 ? (tid / AVPR) * LD + (tid % AVPR) * 16 : st_off;
+  float rsb[2] = {1.f, 1.f};  // weight scales of the tile's two column blocks for the slab in flight
+  const int sb1 = ncols > 128 ? Kd / 128 : 0;  // a tile of one column block reads its scale twice
+  const int st_off_a = (tid / AVPR) * LD + (tid % AVPR) * (AFP8 ? 16 : 8);
+  const int st_off_b = (tid / BVPR) * LD + (tid % BVPR) * (BFP8 ? 16 : 8);
 #define WIDE_FETCH(K0)                                                                           \
   {                                                                                              \
-    const int kv_ = (K0) >> (AFP8 ? 4 : 3);                                                      \
-    _Pragma("unroll") for (int i = 0; i < NA; ++i) ra[i] = xa[offa[i] + kv_];                    \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i) ra[i] = xa[offa[i] + ((K0) >> (AFP8 ? 4 : 3))]; \
     if (AFP8) { _Pragma("unroll") for (int i = 0; i < NS; ++i) rs[i] = xs[offs[i] + ((K0) >> 7)]; } \
-    _Pragma("unroll") for (int i = 0; i < NB; ++i) rb[i] = wb[offb[i] + ((K0) >> 3)];            \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) rb[i] = wb[offb[i] + ((K0) >> (BFP8 ? 4 : 3))]; \
+    if (BFP8) {                                                                                  \
+      rsb[0] = wsc[(K0) >> 7];                                                                   \
+      rsb[1] = wsc[sb1 + ((K0) >> 7)];                                                           \
+    }                                                                                            \
   }
 #define WIDE_STASH(BUF)                                                                                        \
   {                                                                                                            \
     uint16_t* s_a_ = s_wide + (BUF) * (TM + TN) * LD + st_off_a;                                               \
-    uint16_t* s_b_ = s_wide + (BUF) * (TM + TN) * LD + TM * LD + st_off;                                       \
+    uint16_t* s_b_ = s_wide + (BUF) * (TM + TN) * LD + TM * LD + st_off_b;                                     \
     _Pragma("unroll") for (int i = 0; i < NA; ++i) {                                                           \
       if (AFP8) {                                                                                              \
         u32x4_t lo_, hi_;                                                                                      \
@@ -1698,8 +1706,16 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
         *reinterpret_cast<u32x4_t*>(&s_a_[i * (NT / AVPR) * LD]) = ra[i];                                      \
       }                                                                                                        \
     }                                                                                                          \
-    _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                             \
-        *reinterpret_cast<u32x4_t*>(&s_b_[i * (NT / VPR) * LD]) = rb[i];                                       \
+    _Pragma("unroll") for (int i = 0; i < NB; ++i) {                                                           \
+      if (BFP8) { /* vector i sits in row tid / 4 + 64 i: i < NB / 2 is the first column block */              \
+        u32x4_t lo_, hi_;                                                                                      \
+        wide_decode_fp8<E>(rb[i], rsb[i < NB / 2 ? 0 : 1], lo_, hi_);                                          \
+        *reinterpret_cast<u32x4_t*>(&s_b_[i * (NT / BVPR) * LD]) = lo_;                                        \
+        *reinterpret_cast<u32x4_t*>(&s_b_[i * (NT / BVPR) * LD + 8]) = hi_;                                    \
+      } else {                                                                                                 \
+        *reinterpret_cast<u32x4_t*>(&s_b_[i * (NT / BVPR) * LD]) = rb[i];                                      \
+      }                                                                                                        \
+    }                                                                                                          \
   }
 
   f32x16_t acc[WMI][WNJ];
@@ -1728,7 +1744,7 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
   // Instruction classes of the scheduling groups: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read,
   // 0x200 LDS write.  Per step a wave issues MM MFMAs and RD fragment reads, per slab ST stores to
   // LDS and ST global loads.
-  constexpr int RD = WMI + WNJ, MM = WMI * WNJ, ST = (AFP8 ? 2 * NA : NA) + NB;  // LDS stores == global loads
+  constexpr int RD = WMI + WNJ, MM = WMI * WNJ, ST = (AFP8 ? 2 * NA : NA) + (BFP8 ? 2 * NB : NB);  // LDS stores
   constexpr int GW = wide_gcd(MM, ST), GF = wide_gcd(MM - RD, ST - RD);
   static_assert(MM >= RD && ST >= RD, "interleave patterns assume at least one MFMA and one load per read");
 #define WIDE_MIX_READS() /* RD x (LDS read, MFMA), then the other MFMAs */                                      \
@@ -1809,10 +1825,11 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
       }
 }
 
-template <class E, bool AFP8>
+template <class E, bool AFP8, bool BFP8>
 __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const uint4* __restrict__ x,
                                                                          const float* __restrict__ x_scale,
                                                                          const uint4* __restrict__ w,
+                                                                         const float* __restrict__ w_scale,
                                                                          const int32_t* __restrict__ offsets,
                                                                          uint16_t* __restrict__ y, int num_experts,
                                                                          int Kd, int N, int max_recv, int ntile_n) {
@@ -1856,15 +1873,17 @@ __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const ui
   // fp8 rows are Kd bytes (Kd / 16 vectors) with Kd / 128 scales each
   const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * (AFP8 ? Kd / 16 : kvec);
   const float* xs = AFP8 ? x_scale + row0 * (Kd / 128) : nullptr;
-  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * kvec;
+  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * (BFP8 ? Kd / 16 : kvec);
+  // block-quantised weights: N % 128 == 0, the tile's first column block is n0 / 128
+  const float* wsc = BFP8 ? w_scale + ((size_t)e * (N / 128) + n0 / 128) * (Kd / 128) : nullptr;
   uint16_t* y_tile = y + row0 * (size_t)N + n0;
   // A segment's last tile is often less than half full (23 % of the MFMAs of a 512-rows-per-expert
   // ragged input would be spent on rows that do not exist): up to 128 rows the four waves stand
   // side by side on 128 x 64 each, and only 128 rows of A are staged.
   if (rows > 128)
-    wide_tile<E, 4, 4, 256, AFP8>(xa, xs, wb, y_tile, s_wide, rows, ncols, Kd, N, (wave >> 1) * 128, (wave & 1) * 128);
+    wide_tile<E, 4, 4, 256, AFP8, BFP8>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd, N, (wave >> 1) * 128, (wave & 1) * 128);
   else
-    wide_tile<E, 4, 2, 128, AFP8>(xa, xs, wb, y_tile, s_wide, rows, ncols, Kd, N, 0, wave * 64);
+    wide_tile<E, 4, 2, 128, AFP8, BFP8>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd, N, 0, wave * 64);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -2391,9 +2410,11 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   return moe_a2a_combine(expert_y, weights, slot_of_entry, combine_mode, out_type, out, T, K, H, stream);
 }
 
-// Launch of the 256 x 256 kernel; x_scale != nullptr selects fp8 rows of x.
-static int launch_gemm_wide(const void* x, const float* x_scale, const void* weights, const int32_t* offsets, void* y,
-                            int R, int E, int Kd, int N, int max_recv, int elem_type, hipStream_t stream) {
+// Launch of the 256 x 256 kernel; x_scale != nullptr selects fp8 rows of x, w_scale != nullptr
+// block-quantised weights.
+static int launch_gemm_wide(const void* x, const float* x_scale, const void* weights, const float* w_scale,
+                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
+                            hipStream_t stream) {
   const int ntile_n = ceil_div(N, kWideN);
   const long long mtiles = (long long)R / kWideM + E;  // every expert may end with a partly filled tile
   if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
@@ -2405,25 +2426,34 @@ static int launch_gemm_wide(const void* x, const float* x_scale, const void* wei
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= kMaxDevices) return MOE_A2A_E_STATE;
   if (!lds_raised[dev].load(std::memory_order_acquire)) {
-    const void* kernels[4] = {(const void*)expert_gemm_wide_kernel<Bf16, false>,
-                              (const void*)expert_gemm_wide_kernel<F16, false>,
-                              (const void*)expert_gemm_wide_kernel<Bf16, true>,
-                              (const void*)expert_gemm_wide_kernel<F16, true>};
+    const void* kernels[8] = {(const void*)expert_gemm_wide_kernel<Bf16, false, false>,
+                              (const void*)expert_gemm_wide_kernel<F16, false, false>,
+                              (const void*)expert_gemm_wide_kernel<Bf16, true, false>,
+                              (const void*)expert_gemm_wide_kernel<F16, true, false>,
+                              (const void*)expert_gemm_wide_kernel<Bf16, false, true>,
+                              (const void*)expert_gemm_wide_kernel<F16, false, true>,
+                              (const void*)expert_gemm_wide_kernel<Bf16, true, true>,
+                              (const void*)expert_gemm_wide_kernel<F16, true, true>};
     for (const void* k : kernels) {
       hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
       if (e != hipSuccess) return (int)e;
     }
     lds_raised[dev].store(true, std::memory_order_release);
   }
-#define CALL_WIDE(ET, FP8)                                                                                     \
-  return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<ET, FP8>, grid, block, kWideLdsBytes, stream,    \
-                (const uint4*)x, x_scale, (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n)
-  if (x_scale) {
-    if (elem_type == MOE_A2A_BF16) CALL_WIDE(Bf16, true);
-    CALL_WIDE(F16, true);
+#define CALL_WIDE(ET, AF, BF)                                                                                  \
+  return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<ET, AF, BF>, grid, block, kWideLdsBytes, stream, \
+                (const uint4*)x, x_scale, (const uint4*)weights, w_scale, offsets, (uint16_t*)y, E, Kd, N,     \
+                max_recv, ntile_n)
+#define CALL_WIDE_E(ET)                  \
+  {                                      \
+    if (x_scale && w_scale) CALL_WIDE(ET, true, true);  \
+    if (x_scale) CALL_WIDE(ET, true, false);            \
+    if (w_scale) CALL_WIDE(ET, false, true);            \
+    CALL_WIDE(ET, false, false);                        \
   }
-  if (elem_type == MOE_A2A_BF16) CALL_WIDE(Bf16, false);
-  CALL_WIDE(F16, false);
+  if (elem_type == MOE_A2A_BF16) CALL_WIDE_E(Bf16);
+  CALL_WIDE_E(F16);
+#undef CALL_WIDE_E
 #undef CALL_WIDE
 }
 
@@ -2447,7 +2477,7 @@ int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offse
     skinny = atoi(forced) == 32;
   }
   if (Kd % kSkinnyK != 0) skinny = false;  // its K slabs are 128 wide; the 128 x 128 kernel takes the rest
-  if (wide) return launch_gemm_wide(x, nullptr, weights, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
+  if (wide) return launch_gemm_wide(x, nullptr, weights, nullptr, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
   if (skinny) {
     const int ntile_n = ceil_div(N, kSkinnyN);
     const long long mtiles = (long long)R / kSkinnyM + E;
@@ -2481,7 +2511,8 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
   if (R == 0) return 0;
   if (!x_q || !x_scale || !weights || !offsets || !y) return MOE_A2A_E_NULL;
   if (!aligned16(x_q) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
-  return launch_gemm_wide(x_q, x_scale, weights, offsets, y, R, E, Kd, N, max_recv, elem_type, (hipStream_t)stream_);
+  return launch_gemm_wide(x_q, x_scale, weights, nullptr, offsets, y, R, E, Kd, N, max_recv, elem_type,
+                          (hipStream_t)stream_);
 }
 
 int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
@@ -2495,6 +2526,14 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
   if (!x || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
   if (!aligned16(x) || !aligned16(w_q) || !aligned16(y)) return MOE_A2A_E_ALIGN;
   hipStream_t stream = (hipStream_t)stream_;
+  // a decode step streams the weights (32-row tiles); longer segments take the 256 x 256 kernel
+  bool skinny = (long long)R <= 32ll * E || N < kWideN;
+  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) {
+    if (atoi(forced) == 32) skinny = true;
+    if (atoi(forced) == 256 && N >= kWideN) skinny = false;
+  }
+  if (!skinny)
+    return launch_gemm_wide(x, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
   const int ntile_n = N / 128;
   const long long mtiles = (long long)R / kSkinnyM + E;
   if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
