@@ -2041,6 +2041,8 @@ int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_ran
 static int check_rows(const void* a, const void* b, int T, int K, int H, int mult) {
   if (T < 0 || K < 1 || K > MOE_A2A_MAX_TOPK || H < mult || H % mult != 0) return MOE_A2A_E_SHAPE;
   if ((long long)T * K > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
+  // one workgroup per (row, column split) and one more: the grid has to hold them
+  if (((long long)T + 1) * (ceil_div(H / 8, kWave) + 1) > (long long)INT32_MAX) return MOE_A2A_E_SHAPE;
   if (T > 0 && (!a || !b)) return MOE_A2A_E_NULL;
   if (!aligned16(a) || !aligned16(b)) return MOE_A2A_E_ALIGN;
   return 0;
@@ -2558,8 +2560,19 @@ int moe_a2a_timer_begin(int capacity) {
   g_timer.ids = new int[capacity];
   for (int i = 0; i < capacity; ++i) {
     hipError_t e1 = hipEventCreate(&g_timer.start[i]);
-    hipError_t e2 = hipEventCreate(&g_timer.stop[i]);
-    if (e1 != hipSuccess || e2 != hipSuccess) return (int)(e1 != hipSuccess ? e1 : e2);
+    hipError_t e2 = e1 == hipSuccess ? hipEventCreate(&g_timer.stop[i]) : e1;
+    if (e2 != hipSuccess) {  // give back what exists: events 0 .. i-1 in pairs, and start[i] if it was made
+      if (e1 == hipSuccess) (void)hipEventDestroy(g_timer.start[i]);
+      for (int j = 0; j < i; ++j) {
+        (void)hipEventDestroy(g_timer.start[j]);
+        (void)hipEventDestroy(g_timer.stop[j]);
+      }
+      delete[] g_timer.start;
+      delete[] g_timer.stop;
+      delete[] g_timer.ids;
+      g_timer = LaunchTimer{};
+      return (int)e2;
+    }
   }
   g_timer.capacity = capacity;
   g_timer.used = 0;
