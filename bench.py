@@ -347,7 +347,7 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
         e1.record(main)
         main.synchronize()
     ms_step = e0.elapsed_time(e1) / args.steps
-    kernel = next(k for k in ("expert_gemm_wide", "expert_gemm_skinny", "expert_gemm") if k in per)
+    kernel = next(k for k in ("expert_gemm_f8", "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm") if k in per)
     t_us = statistics.fmean(per[kernel])
     flops = 2.0 * R * H * N
     tflops = flops / t_us / 1e6
