@@ -212,16 +212,20 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
  * w_q[E, N, Kd] e4m3fn bytes with w_scale[E, N/128, Kd/128] f32 (one scale per 128 x 128 block).
  * x is 16-bit (x_scale == NULL) or the e4m3fn rows + x_scale[rows, Kd/128] of moe_a2a_dispatch_fp8
  * (dequantised and rounded once to elem_type inside the kernel); y[rows, N] of elem_type.
- * Kd % 128 == 0, N % 128 == 0.  Two kernels, chosen by the mean segment length:
+ * Kd % 128 == 0, N % 128 == 0.  Three kernels, chosen by the mean segment length and the rows:
  *   R <= 32 * E (a decode step, bound by the weight bytes, which cross memory once at one byte per
- *     element): 32 x 128 tiles; the weight bytes enter the matrix cores exactly, each 128-wide K
- *     block is summed in f32 and scaled in f32: y = sum over K blocks of scale_b * (x . q_b).
- *   longer segments (and N >= 256): the 256 x 256 kernel; a weight enters the matrix cores as
- *     elem(f32(q) * scale), i.e. dequantised and rounded once to elem_type on its way into LDS --
- *     the result of dequantising the weights to 16 bits and calling moe_a2a_expert_gemm, without
- *     the 16-bit copy in memory.
- * The two differ by that one rounding of a weight (2^-9 relative for bf16); MOE_A2A_GEMM_TILE=32 or
- * 256 forces one.  No counterpart in the reference.
+ *     element): 32 x 128 tiles; the weight bytes enter the matrix cores exactly (as 16-bit values),
+ *     each 128-wide K block is summed in f32 and scaled in f32: y = sum over K blocks of
+ *     scale_b * (x . q_b); fp8 rows are dequantised and rounded once to elem_type first.
+ *   longer segments, fp8 rows: both operands enter the fp8 matrix instruction as bytes
+ *     (v_mfma_f32_32x32x64_f8f6f4), each 128-wide K block is summed in f32 and folded with
+ *     x_scale[row][kb] * w_scale[n / 128][kb]; nothing is rounded before the output.
+ *   longer segments, 16-bit rows (and N >= 256): the 256 x 256 kernel; a weight enters the matrix
+ *     cores as elem(f32(q) * scale), i.e. dequantised and rounded once to elem_type on its way into
+ *     LDS -- the result of dequantising the weights to 16 bits and calling moe_a2a_expert_gemm,
+ *     without the 16-bit copy in memory.
+ * The three differ by those roundings (2^-9 relative per operand for bf16); MOE_A2A_GEMM_TILE=32,
+ * 128 (fp8 rows) or 256 forces one.  No counterpart in the reference.
  */
 int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,

@@ -1921,8 +1921,8 @@ __global__ __launch_bounds__(2 * TN, TN == 128 ? 2 : 1) void expert_gemm_f8_kern
                                                                        int Kd, int N, int max_recv, int ntile_n) {
   constexpr int TM = kF8M, BK = kF8K, LD = kF8Ld, NT = 2 * TN;  // a wave per 64 x 64 corner of the tile
   constexpr int NA = TM * 8 / NT, NB = TN * 8 / NT;               // vectors of a slab per thread
-  __shared__ __attribute__((aligned(16))) uint8_t s_ab8[2 * (TM + TN) * LD];  // two slabs
-  __shared__ __attribute__((aligned(16))) float s_sx[2 * TM];                 // row scales of each
+  __shared__ __attribute__((aligned(16))) uint8_t s_ab8[(TM + TN) * LD];  // the slab
+  __shared__ __attribute__((aligned(16))) float s_sx[TM];                 // its row scales
   __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
   __shared__ int s_tmp[NT / kWave + 1];
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -1966,10 +1966,10 @@ __global__ __launch_bounds__(2 * TN, TN == 128 ? 2 : 1) void expert_gemm_f8_kern
   const int n0 = tile_n * TN;  // N % TN == 0
   const int kvec = Kd / 16, kblk = Kd / BK;
 
-  // global -> register prefetch: a slab is 128 + 128 rows of 8 vectors, four + four per thread,
-  // one row scale for each of the first 128 threads, one weight scale (uniform).  Two register
-  // sets and two LDS buffers: a slab is requested two iterations before it is multiplied and is
-  // written into the buffer the current slab does not use; one barrier per slab.
+  // global -> register prefetch: a slab is 128 + TN rows of 8 vectors per row, one row scale for
+  // each of the first 128 threads, one weight scale (uniform over the wave).  (Two register sets
+  // and two LDS buffers, a slab requested two iterations ahead, measured 2 % faster and leave no
+  // register for the loop specialisation below.)
   const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x_q) + row0 * kvec;
   const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w_q) + ((size_t)e * N + n0) * kvec;
   const float* xs = x_scale + (row0 + min(tid, rows - 1)) * kblk;
@@ -1980,7 +1980,7 @@ __global__ __launch_bounds__(2 * TN, TN == 128 ? 2 : 1) void expert_gemm_f8_kern
     u32x4_t a[NA], b[NB];
     float sx, sw;
   };
-  Slab r0, r1;
+  Slab r0;
   int offa[NA], offb[NB];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
@@ -2020,60 +2020,66 @@ __global__ __launch_bounds__(2 * TN, TN == 128 ? 2 : 1) void expert_gemm_f8_kern
       for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
   const int fr_a = (wm + (lane & 31)) * LD + (lane >> 5) * 32;
   const int fr_b = (TM + wn + (lane & 31)) * LD + (lane >> 5) * 32;
+  // 32-row blocks of this wave that hold rows of the segment: 0, 1 or 2 (uniform over the wave)
+  const int live_blocks = __builtin_amdgcn_readfirstlane(min(2, max(0, (rows - wm + 31) / 32)));
 
-#define F8_SLAB(BUF, S)                                                                                         \
+#define F8_SLAB(BUF, S, LB)                                                                                     \
   {                                                                                                            \
     const uint8_t* sb_ = s_ab8 + (BUF) * (TM + TN) * LD;                                                       \
     f32x16_t part[2][2];                                                                                       \
     _Pragma("unroll") for (int kk = 0; kk < BK; kk += 64) {                                                    \
       i32x8_t fa[2], fb[2];                                                                                    \
       _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                          \
-        const u32x4_t a0 = *reinterpret_cast<const u32x4_t*>(&sb_[fr_a + i * 32 * LD + kk]);                   \
-        const u32x4_t a1 = *reinterpret_cast<const u32x4_t*>(&sb_[fr_a + i * 32 * LD + kk + 16]);              \
         const u32x4_t b0 = *reinterpret_cast<const u32x4_t*>(&sb_[fr_b + i * 32 * LD + kk]);                   \
         const u32x4_t b1 = *reinterpret_cast<const u32x4_t*>(&sb_[fr_b + i * 32 * LD + kk + 16]);              \
-        fa[i] = i32x8_t{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3],                                        \
-                        (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};                                       \
         fb[i] = i32x8_t{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3],                                        \
                         (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};                                       \
       }                                                                                                        \
       _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                            \
-      _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                          \
-        f32x16_t zero;                                                                                         \
-        _Pragma("unroll") for (int q = 0; q < 16; ++q) zero[q] = 0.f;                                          \
-        part[i][j] = mfma_32x32x64_fp8(fb[j], fa[i], kk == 0 ? zero : part[i][j]); /* weights x rows^T */      \
+        if (i < (LB)) { /* blocks of 32 rows past the segment cost no MFMA */                                  \
+          const u32x4_t a0 = *reinterpret_cast<const u32x4_t*>(&sb_[fr_a + i * 32 * LD + kk]);                 \
+          const u32x4_t a1 = *reinterpret_cast<const u32x4_t*>(&sb_[fr_a + i * 32 * LD + kk + 16]);            \
+          fa[i] = i32x8_t{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3],                                      \
+                          (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};                                     \
+          _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                      \
+            f32x16_t zero;                                                                                     \
+            _Pragma("unroll") for (int q = 0; q < 16; ++q) zero[q] = 0.f;                                      \
+            part[i][j] = mfma_32x32x64_fp8(fb[j], fa[i], kk == 0 ? zero : part[i][j]); /* weights x rows^T */  \
+          }                                                                                                    \
+        }                                                                                                      \
+    }                                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                              \
+      if (i < (LB)) {                                                                                          \
+        /* the lane's row of x: one factor for all 16 elements, row scale x weight scale */                    \
+        const float sc = s_sx[(BUF) * TM + wm + i * 32 + (lane & 31)] * S;                                     \
+        _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                          \
+        _Pragma("unroll") for (int q = 0; q < 16; ++q)                                                         \
+            acc[i][j][q] = __builtin_fmaf(part[i][j][q], sc, acc[i][j][q]);                                    \
       }                                                                                                        \
-    }                                                                                                          \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                            \
-      /* the lane's row of x: one factor for all 16 elements, row scale x weight scale */                      \
-      const float sc = s_sx[(BUF) * TM + wm + i * 32 + (lane & 31)] * S;                                       \
-      _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                            \
-      _Pragma("unroll") for (int q = 0; q < 16; ++q)                                                           \
-          acc[i][j][q] = __builtin_fmaf(part[i][j][q], sc, acc[i][j][q]);                                      \
-    }                                                                                                          \
   }
 
-  // slab kb is multiplied from buffer kb & 1; slab kb + 1 waits in one register set and goes into
-  // the other buffer at the end of the iteration; slab kb + 2 is requested at its start.  The
-  // weight scale of a slab stays in a register of its own until the slab has been folded.
-  F8_FETCH(r0, 0);
-  F8_FETCH(r1, 1);
-  F8_STASH(r0, 0);
-  float sw0 = r0.sw, sw1;
-  __syncthreads();
-  for (int kb = 0; kb < kblk; kb += 2) {
-    F8_FETCH(r0, kb + 2);
-    F8_SLAB(0, sw0);
-    F8_STASH(r1, 1);
-    sw1 = r1.sw;
-    __syncthreads();
-    if (kb + 1 >= kblk) break;
-    F8_FETCH(r1, kb + 3);
-    F8_SLAB(1, sw1);
-    F8_STASH(r0, 0);
-    sw0 = r0.sw;
-    __syncthreads();
+  // Per slab: registers -> LDS, barrier, request the next slab (in flight during the multiplies),
+  // multiply and fold, barrier.  The loop exists three times, for waves with two, one and no 32-row
+  // block inside the segment (a wave without rows still moves its share of every slab and meets
+  // every barrier): at 128 rows per expert on average a third of all 32-row blocks are empty.
+#define F8_LOOP(LB)                              \
+  for (int kb = 0; kb < kblk; ++kb) {            \
+    F8_STASH(r0, 0);                             \
+    const float sw = r0.sw;                      \
+    __syncthreads();                             \
+    F8_FETCH(r0, kb + 1);                        \
+    F8_SLAB(0, sw, LB);                          \
+    __syncthreads();                             \
   }
+  F8_FETCH(r0, 0);
+  if (live_blocks == 2) {
+    F8_LOOP(2)
+  } else if (live_blocks == 1) {
+    F8_LOOP(1)
+  } else {
+    F8_LOOP(0)
+  }
+#undef F8_LOOP
 #undef F8_SLAB
 #undef F8_STASH
 #undef F8_FETCH
@@ -2739,15 +2745,22 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
   if (!x || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
   if (!aligned16(x) || !aligned16(w_q) || !aligned16(y)) return MOE_A2A_E_ALIGN;
   hipStream_t stream = (hipStream_t)stream_;
-  // a decode step streams the weights (32-row tiles); longer segments take the 256 x 256 kernel
-  bool skinny = (long long)R <= 32ll * E || (N < kWideN && !x_scale);
+  // A decode step streams the weights (32-row tiles); longer segments multiply fp8 by fp8 when the
+  // rows are fp8, else on the 256 x 256 kernel, which dequantises the weights on their way into LDS
+  // (it needs N >= 256).  MOE_A2A_GEMM_TILE = 32 | 128 | 256 forces one where it applies.
+  enum { kStream, kBothFp8, kDequant } kernel;
+  if ((long long)R <= 32ll * E) kernel = kStream;
+  else if (x_scale) kernel = kBothFp8;
+  else kernel = N >= kWideN ? kDequant : kStream;
   if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) {
-    if (atoi(forced) == 32) skinny = true;
-    if (atoi(forced) == 128 && x_scale) skinny = false;
-    if (atoi(forced) == 256 && N >= kWideN) skinny = false;
-    if (atoi(forced) == 256 && N < kWideN && !x_scale) skinny = true;
+    const int tile = atoi(forced);
+    if (tile == 32) kernel = kStream;
+    if (tile == 128 && x_scale) kernel = kBothFp8;
+    if (tile == 256 && N >= kWideN) kernel = kDequant;
   }
-  if (!skinny && x_scale && !(getenv("MOE_A2A_GEMM_TILE") && atoi(getenv("MOE_A2A_GEMM_TILE")) == 256)) {
+  if (kernel == kDequant)
+    return launch_gemm_wide(x, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
+  if (kernel == kBothFp8) {
     // both operands fp8: the bytes go to the matrix cores as they are.  128 x 128 tiles: the
     // 128 x 256 form of the kernel (one workgroup of eight waves per CU) measured slower, 1160
     // against 1140 us at 128 rows per expert and 1030 against 920 us at 512.
@@ -2763,8 +2776,6 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
     return launch(KID_EXPERT_GEMM_F8, expert_gemm_f8_kernel<F16, tn>, grid, block, 0, stream, (const uint4*)x,
                   x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
   }
-  if (!skinny)
-    return launch_gemm_wide(x, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
   const int ntile_n = N / 128;
   const long long mtiles = (long long)R / kSkinnyM + E;
   if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;

@@ -23,7 +23,7 @@ per (row, 128-column block) ``amax = max|f32(x)|``, ``scale = amax / 448`` in f3
 PARITY UNPINNED against the reference for that function (nothing to pin against);
 it is pinned against torch's own e4m3fn cast and the stated error bound only.
 
-``expert_gemm`` / ``expert_gemm_fp8`` (a per-expert linear layer in place of the stub) have no
+``expert_gemm`` / ``expert_gemm_fp8`` / ``expert_gemm_q8`` (a per-expert linear layer in place of the stub) have no
 counterpart in the reference either: PARITY UNPINNED against it; they are an f32 torch matmul per
 segment and serve as the tolerance reference for the HIP grouped GEMM.
 """
@@ -176,14 +176,20 @@ def dequantize_weights_fp8(q_bits: torch.Tensor, scale: torch.Tensor) -> torch.T
 
 
 def expert_gemm_q8(disp_x: torch.Tensor, x_scale, w_bits: torch.Tensor, w_scale: torch.Tensor,
-                   offsets: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+                   offsets: torch.Tensor, out_dtype: torch.dtype, round_rows: bool = True) -> torch.Tensor:
     """The expert layer with block-quantised weights: ``y = sum over K blocks of scale_b * (x . q_b)``,
     i.e. the weights enter exactly (``f32(q) * scale`` in f32) and everything is summed in f32, one
-    rounding to ``out_dtype`` at the end.  fp8 rows (``x_scale`` given) are dequantised and rounded
-    once to ``out_dtype`` first, as in ``expert_gemm_fp8``.  No counterpart in the reference:
-    PARITY UNPINNED against it."""
+    rounding to ``out_dtype`` at the end.  fp8 rows (``x_scale`` given) are dequantised and, with
+    ``round_rows``, rounded once to ``out_dtype`` first, as in ``expert_gemm_fp8`` (the kernels that
+    multiply on the 16-bit matrix instruction do that); without it they enter as ``f32(q) * scale``
+    (the kernel that multiplies fp8 by fp8 rounds nothing before the output).  No counterpart in the
+    reference: PARITY UNPINNED against it."""
     w = dequantize_weights_fp8(w_bits, w_scale)  # f32
-    x = dequantize_fp8(disp_x, x_scale).to(out_dtype) if x_scale is not None else disp_x
+    if x_scale is None:
+        x = disp_x
+    else:
+        x = dequantize_fp8(disp_x, x_scale)
+        x = x.to(out_dtype) if round_rows else x
     R = x.shape[0]
     E, N, _ = w.shape
     y = torch.zeros(R, N, dtype=out_dtype)
