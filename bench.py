@@ -64,6 +64,7 @@ def parse_args():
     p.add_argument("--expert-gemm", type=int, default=0, metavar="N",
                    help="measure the grouped expert GEMM (N output columns per expert) on the workload's "
                         "dispatched rows instead of the dispatch/combine path")
+    p.add_argument("--dump-times", metavar="FILE", help="write every timed launch's duration (us, in launch order) as JSON")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="end with three plain 256 MiB device copies (a known-size reference for rocprof counters)")
     return p.parse_args()
@@ -211,6 +212,9 @@ def main():
         # (creating them costs driver calls that land in the middle of the launch sequence)
         kernel_times(lib, run_n, args.steps, torch)
         per = kernel_times(lib, run_n, args.steps, torch)
+        if args.dump_times:
+            with open(args.dump_times, "w") as f:
+                json.dump(per, f)
         e0.record(main)
         run_n(timed_steps)
         e1.record(main)
@@ -443,11 +447,28 @@ def cpu_baseline(wl, mode, fp8, y_gpu, b_dc, budget_s):
             break
     us = statistics.median(times[1:])
     same = bool(torch.equal(y_gpu.cpu().view(torch.int16), y_cpu.view(torch.int16)))
-    return dict(value=round(b_dc / us / 1e3, 3), unit="GB/s", cores=torch.get_num_threads(), kind="port",
-                dispatch_combine_us=round(us, 1),
-                sample=f"full workload {wl.name}: {len(times) - 1} timed passes of route+dispatch+combine "
-                       f"(vectorised torch-CPU oracle), median",
-                gpu_output_bit_identical=same)
+    out = dict(value=round(b_dc / us / 1e3, 3), unit="GB/s", cores=torch.get_num_threads(), kind="port",
+               dispatch_combine_us=round(us, 1),
+               sample=f"full workload {wl.name}: {len(times) - 1} timed passes of route+dispatch+combine "
+                      f"(vectorised torch-CPU oracle), median",
+               gpu_output_bit_identical=same)
+    # the row-by-row form of the reference's loops (all2all/reference.py:123-146, 227-232), where it
+    # finishes in a second: three passes, median; fp8 has no row-loop form
+    if not fp8 and mode == 0 and x.shape[0] * K <= 8192:
+        from oracle import all2all_literal as Lit
+
+        lit = []
+        for _ in range(3):
+            t0 = time.perf_counter_ns()
+            disp = Lit.dispatch_world(cfg, wl.world)
+            t1 = time.perf_counter_ns()
+            ey = Lit.stub_world(cfg, disp, wl.stub_kind)
+            t2 = time.perf_counter_ns()
+            Lit.combine_world(cfg, wl.world, disp, ey)
+            t3 = time.perf_counter_ns()
+            lit.append(((t1 - t0) + (t3 - t2)) / 1e3)
+        out["row_loop_dispatch_combine_us"] = round(statistics.median(lit), 1)
+    return out
 
 
 if __name__ == "__main__":
