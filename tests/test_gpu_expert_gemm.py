@@ -269,3 +269,53 @@ def test_expert_gemm_argument_checks(gpu_device):
     from kernel_amd._lib import MoeA2AError
     with pytest.raises(MoeA2AError):  # hidden size must be a multiple of 64
         bad.expert_gemm(db, torch.zeros(8, 64, 72, dtype=torch.bfloat16, device=gpu_device))
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_shapes_every_expert_gemm_form(gpu_device, monkeypatch, seed):
+    """Seeded sweep: random expert counts, segment lengths (empty experts, segments that end a
+    row or two past a tile), hidden and output sizes, layouts, element types, and every operand
+    format (16-bit, fp8 rows, fp8 block-quantised weights, both) through whichever kernel the
+    library picks for the shape and, on odd seeds, through a forced one."""
+    g = torch.Generator().manual_seed(1000 + seed)
+
+    def pick(options):
+        return options[int(torch.randint(len(options), (1,), generator=g))]
+
+    E = pick([1, 3, 8, 9, 24, 40])
+    K = pick([1, 2, 4])
+    K = min(K, E)
+    T = pick([1, 7, 33, 129, 260, 600, 1100])
+    H = pick([128, 256, 384, 640])
+    N = pick([128, 256, 384, 512, 640])
+    W = pick([w for w in (1, 2, 4, 8) if E % w == 0])
+    dtype = pick([torch.bfloat16, torch.float16])
+    zipf = pick([False, True])
+    padded = pick([False, True])
+    fp8_rows = pick([False, True])
+    q8 = pick([False, True])
+    if seed % 2:
+        monkeypatch.setenv("MOE_A2A_GEMM_TILE", pick(["32", "128", "256"]))
+    else:
+        monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
+    cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=seed, zipf=zipf)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, fp8_dispatch=fp8_rows, padded=padded, max_recv=T if padded else None)
+    d = ata.dispatch(x, idx, rs)
+    o = V.run_world(cfg, world, fp8=fp8_rows)
+    if q8:
+        wq, ws = V.quantize_weights_fp8(weights)
+        y = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device))
+        # which of the q8 kernels ran decides whether fp8 rows were rounded to 16 bits first; both
+        # readings of the rows differ by far less than the tolerance, so the unrounded one serves
+        want = V.expert_gemm_q8(o["disp_x"], o["disp_scale"] if fp8_rows else None, wq, ws, o["offsets"], dtype,
+                                round_rows=False)
+    elif fp8_rows:
+        y = ata.expert_gemm(d, weights.to(gpu_device))
+        want = V.expert_gemm_fp8(o["disp_x"], o["disp_scale"], o["offsets"], weights, dtype)
+    else:
+        y = ata.expert_gemm(d, weights.to(gpu_device))
+        want = V.expert_gemm(o["disp_x"], o["offsets"], weights, dtype)
+    torch.cuda.synchronize()
+    rows = d.slot_of_entry.long() if padded else o["slot_of_entry"].long().to(gpu_device)
+    close(y[rows], want[o["slot_of_entry"].long()])
