@@ -61,6 +61,10 @@ def parse_args():
     p.add_argument("--cpu-seconds", type=float, default=12.0)
     p.add_argument("--fp8-weights", action="store_true",
                    help="with --expert-gemm: weights as e4m3fn bytes with one f32 scale per 128 x 128 block")
+    p.add_argument("--fp8-rows", action="store_true", help="with --expert-gemm: fp8 dispatch on a 16-bit workload")
+    p.add_argument("--pow2-scales", action="store_true",
+                   help="with --expert-gemm --fp8-weights on an fp8 workload: power-of-two scales for rows and weights, "
+                        "multiplied with the scales as the matrix instruction's block exponents")
     p.add_argument("--expert-gemm", type=int, default=0, metavar="N",
                    help="measure the grouped expert GEMM (N output columns per expert) on the workload's "
                         "dispatched rows instead of the dispatch/combine path")
@@ -325,8 +329,11 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
 
     cfg = wl.cfg
     E, H, N = cfg.num_experts, cfg.hidden_dim, args.expert_gemm
-    fp8 = wl.fp8_dispatch and not args.bf16_dispatch  # fp8 rows are dequantised inside the kernel
-    ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fp8_dispatch=fp8)
+    fp8 = (wl.fp8_dispatch or args.fp8_rows) and not args.bf16_dispatch
+    pow2 = bool(args.pow2_scales)
+    if pow2 and not (fp8 and args.fp8_weights):
+        raise SystemExit("--pow2-scales needs an fp8 workload (fp8 rows) and --fp8-weights")
+    ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fp8_dispatch="pow2" if pow2 else fp8)
     gen = torch.Generator(device="cpu").manual_seed(1234)
     weights = (torch.randn(E, N, H, generator=gen) / H ** 0.5).to(cfg.in_dtype).to(dev)
     w_scale = None
@@ -334,6 +341,9 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
         wf = weights.float().view(E, N // 128, 128, H // 128, 128)
         amax = wf.abs().amax(dim=(2, 4))
         w_scale = torch.where(amax == 0, torch.ones_like(amax), amax / 448.0).contiguous()
+        if pow2:  # the next power of two at or above (exponent field + 1 when the mantissa is not zero)
+            u = w_scale.view(torch.int32)
+            w_scale = (((u >> 23) + ((u & 0x7FFFFF) != 0).to(torch.int32)).clamp(1, 254) << 23).view(torch.float32)
         weights = (wf / w_scale[:, :, None, :, None]).to(torch.float8_e4m3fn).view(E, N, H).contiguous()
     main = torch.cuda.Stream()
     main.wait_stream(torch.cuda.current_stream())
@@ -342,17 +352,17 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
         R = d.num_rows
         y = torch.empty(R, N, dtype=cfg.in_dtype, device=dev)
         for _ in range(args.warmup):
-            ata.expert_gemm(d, weights, out=y, w_scale=w_scale)
+            ata.expert_gemm(d, weights, out=y, w_scale=w_scale, scales_pow2=pow2)
         main.synchronize()
-        per = kernel_times(lib, lambda n: [ata.expert_gemm(d, weights, out=y, w_scale=w_scale) for _ in range(n)], args.steps, torch)
+        per = kernel_times(lib, lambda n: [ata.expert_gemm(d, weights, out=y, w_scale=w_scale, scales_pow2=pow2) for _ in range(n)], args.steps, torch)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(main)
         for _ in range(args.steps):
-            ata.expert_gemm(d, weights, out=y, w_scale=w_scale)
+            ata.expert_gemm(d, weights, out=y, w_scale=w_scale, scales_pow2=pow2)
         e1.record(main)
         main.synchronize()
     ms_step = e0.elapsed_time(e1) / args.steps
-    kernel = next(k for k in ("expert_gemm_f8", "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm") if k in per)
+    kernel = next(k for k in ("expert_gemm_mx", "expert_gemm_f8", "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm") if k in per)
     t_us = statistics.fmean(per[kernel])
     flops = 2.0 * R * H * N
     tflops = flops / t_us / 1e6
@@ -369,8 +379,8 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
     # the output); if that takes longer at 8 TB/s than the flops at the MFMA peak, the launch is HBM-bound
     live = int((d.counts > 0).sum())
     # the kernel with both operands fp8 multiplies on the fp8 matrix instruction (dense peak 5.0 PFLOP/s)
-    mfma_peak = FP8_MFMA_PEAK_TFLOPS if kernel == "expert_gemm_f8" else MFMA_PEAK_TFLOPS
-    if kernel == "expert_gemm_f8":
+    mfma_peak = FP8_MFMA_PEAK_TFLOPS if kernel in ("expert_gemm_f8", "expert_gemm_mx") else MFMA_PEAK_TFLOPS
+    if kernel in ("expert_gemm_f8", "expert_gemm_mx"):
         out["dtype"] = "fp8"
     gemm_bytes = R * H * (1 + 4 / 128 if fp8 else 2) + live * N * H * (1 if args.fp8_weights else 2) + R * N * 2
     if gemm_bytes / (HBM_PEAK_GBPS * 1e3) > flops / (mfma_peak * 1e6):

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MOE_A2A_ABI_VERSION 2
+#define MOE_A2A_ABI_VERSION 3
 
 /* element types of activations */
 #define MOE_A2A_F16 0
@@ -50,6 +50,9 @@ extern "C" {
 #define MOE_A2A_MAX_WORLD 256
 #define MOE_A2A_META_DIM 5
 #define MOE_A2A_FP8_BLOCK 128
+/* scale of an fp8 block: amax / 448 in f32, or that rounded up to a power of two */
+#define MOE_A2A_FP8_SCALE_F32 0
+#define MOE_A2A_FP8_SCALE_POW2 1
 
 /* argument errors */
 #define MOE_A2A_E_NULL (-1)      /* a required pointer is NULL                       */
@@ -129,10 +132,14 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
  * (scale = amax/448, 1 if amax == 0; q = rne_e4m3(x / scale)), then store row and scales at
  * the K slots.  x is MOE_A2A_F16 or MOE_A2A_BF16, H % 128 == 0.  The reference has no fp8
  * path; the arithmetic is the one stated here.
+ *   scale_mode  MOE_A2A_FP8_SCALE_F32: scale as above.  MOE_A2A_FP8_SCALE_POW2: that value rounded
+ *               up to the next power of two (exponent field clamped to 1..254), still stored as
+ *               f32 -- every consumer of the rows works unchanged, and moe_a2a_expert_gemm_mx8 can
+ *               hand the exponents to the matrix instruction.
  *   disp_q[R,H] uint8, disp_scale[R,H/128] f32
  */
 int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry, uint8_t* disp_q,
-                         float* disp_scale, int T, int K, int H, moe_a2a_stream_t stream);
+                         float* disp_scale, int T, int K, int H, int scale_mode, moe_a2a_stream_t stream);
 
 /*
  * Expert stub (all2all/reference.py:262): y[row,:] = round_out(f32(round_out(x[row,:])) * s(e)),
@@ -168,7 +175,8 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
  * does between reading its inputs and returning y (submission.py:192-219 of the reference;
  * ref_kernel, all2all/reference.py:256-272).  Same kernels and results as the separate calls;
  * one host call keeps the launches back to back.
- *   fp8_dispatch  0 / 1          fuse_stub  0: stub kernel + combine, 1: moe_a2a_stub_combine
+ *   fp8_dispatch  0: 16-bit rows, 1: fp8 rows with f32 scales, 2: fp8 rows with power-of-two scales
+ *   fuse_stub     0: stub kernel + combine, 1: moe_a2a_stub_combine
  *   fuse_route    0: moe_a2a_route + dispatch, 1: moe_a2a_route_dispatch when moe_a2a_fused_ok,
  *                 2: moe_a2a_route_dispatch at any size
  *   expert_y      [R,H] (padded layout: [E*max_recv,H]) of out_type, unused (may be NULL) when fuse_stub
@@ -230,6 +238,23 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
 int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
                            moe_a2a_stream_t stream);
+
+/*
+ * The same product for operands whose scales are all powers of two (rows from moe_a2a_dispatch_fp8
+ * with MOE_A2A_FP8_SCALE_POW2, weights quantised with power-of-two block scales, the UE8M0 style
+ * of newer DeepSeek checkpoints): on long segments (R >= 256 * E) the bytes of both operands go
+ * to v_mfma_scale_f32_32x32x64_f8f6f4 and the exponent fields of the scales ride along as the
+ * instruction's block exponents, so the products of all K blocks accumulate inside the matrix
+ * cores (256 x 256 tiles, nothing is folded on the vector units).  y = sum over K blocks of
+ * x_scale * w_scale * (q_x . q_w) in f32, one rounding to elem_type.  ONLY the exponent field of a
+ * scale is used: a scale that is not a power of two is silently taken as the power of two below
+ * it.  Shorter segments go through moe_a2a_expert_gemm_q8 (any f32 scale; MOE_A2A_GEMM_TILE=256
+ * forces the tiles).  Arguments as for
+ * moe_a2a_expert_gemm_q8 with x_scale required.  No counterpart in the reference.
+ */
+int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w_q, const float* w_scale,
+                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
+                            moe_a2a_stream_t stream);
 
 /*
  * Launch timer (opt-in, process-wide, single caller thread).  Between begin and end every

@@ -9,8 +9,9 @@ import os
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmoe_a2a.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 F16, BF16 = 0, 1
+FP8_SCALE_F32, FP8_SCALE_POW2 = 0, 1
 
 _i32p = C.c_void_p  # device pointers travel as plain addresses
 _vp = C.c_void_p
@@ -28,7 +29,7 @@ PROTOTYPES = {
     "moe_a2a_fused_ok": (_int, [_int, _int, _int]),
     "moe_a2a_route_dispatch": (_int, [_vp, _i32p, _i32p, _int, _int, _int, _int, _int, _int, _int, _i32p, _i32p,
                                       _i32p, _i32p, _i32p, _i32p, _vp, _vp]),
-    "moe_a2a_dispatch_fp8": (_int, [_vp, _int, _i32p, _vp, _vp, _int, _int, _int, _vp]),
+    "moe_a2a_dispatch_fp8": (_int, [_vp, _int, _i32p, _vp, _vp, _int, _int, _int, _int, _vp]),
     "moe_a2a_stub": (_int, [_vp, _vp, _i32p, _i32p, _int, _int, _int, _int, _int, _vp, _int, _int, _vp]),
     "moe_a2a_combine": (_int, [_vp, _vp, _i32p, _int, _int, _vp, _int, _int, _int, _vp]),
     "moe_a2a_stub_combine": (_int, [_vp, _vp, _i32p, _vp, _i32p, _int, _int, _int, _int, _int, _int, _vp, _int, _int,
@@ -38,6 +39,7 @@ PROTOTYPES = {
     "moe_a2a_expert_gemm": (_int, [_vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_expert_gemm_fp8": (_int, [_vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_expert_gemm_q8": (_int, [_vp, _vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
+    "moe_a2a_expert_gemm_mx8": (_int, [_vp, _vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_timer_begin": (_int, [_int]),
     "moe_a2a_timer_end": (_int, [C.POINTER(C.c_int), C.POINTER(C.c_float), _int]),
     "moe_a2a_kernel_name": (C.c_char_p, [_int]),

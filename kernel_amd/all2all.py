@@ -118,6 +118,10 @@ class HipAllToAll:
         self.padded = padded  # rows laid out as the reference's [E_l, max_recv, .] buffers of every owner rank
         self.stub_kind = stub_kind
         self.combine_mode = combine_mode
+        # False: 16-bit rows; True: fp8 rows with f32 scales (amax / 448); "pow2": fp8 rows whose scales
+        # are that rounded up to a power of two (what expert_gemm(..., scales_pow2=True) needs)
+        if fp8_dispatch not in (False, True, "pow2"):
+            raise ValueError("fp8_dispatch is False, True or 'pow2'")
         self.fp8_dispatch = fp8_dispatch
         self.fuse_route = fuse_route
         self.fuse_stub = fuse_stub
@@ -208,7 +212,9 @@ class HipAllToAll:
                                          _ptr(b["workspace"]), b["workspace"].numel(), st), "moe_a2a_route")
             if self.fp8_dispatch:
                 _lib.check(lib.moe_a2a_dispatch_fp8(_ptr(dp_x), _elem(cfg.in_dtype), _ptr(b["slot_of_entry"]),
-                                                    _ptr(b["disp_x"]), _ptr(b["disp_scale"]), T, K, H, st),
+                                                    _ptr(b["disp_x"]), _ptr(b["disp_scale"]), T, K, H,
+                                                    _lib.FP8_SCALE_POW2 if self.fp8_dispatch == "pow2"
+                                                    else _lib.FP8_SCALE_F32, st),
                            "moe_a2a_dispatch_fp8")
             else:
                 _lib.check(lib.moe_a2a_dispatch(_ptr(dp_x), _ptr(b["slot_of_entry"]), _ptr(b["disp_x"]), T, K, H, st),
@@ -230,7 +236,7 @@ class HipAllToAll:
         return y
 
     def expert_gemm(self, d: Dispatched, weights: torch.Tensor, out: Optional[torch.Tensor] = None,
-                    w_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    w_scale: Optional[torch.Tensor] = None, scales_pow2: bool = False) -> torch.Tensor:
         """Real expert compute in place of the stub: ``y[rows of e] = disp_x[rows of e] @ weights[e].T``
         for every expert, on the matrix cores (f32 accumulation, one rounding to ``out_dtype``).
 
@@ -241,6 +247,11 @@ class HipAllToAll:
 
         Block-quantised weights: ``weights`` as e4m3fn bits (``uint8`` or ``float8_e4m3fn``) with
         ``w_scale[E, N/128, H/128]`` f32, the format of DeepSeek-V3 checkpoints; ``N % 128 == 0``.
+
+        ``scales_pow2``: the caller states that every scale of both operands is a power of two
+        (rows from ``fp8_dispatch="pow2"``, weights quantised that way); the library then hands the
+        scales' exponents to the matrix instruction (``moe_a2a_expert_gemm_mx8``).  Only the exponent
+        field of a scale is used there, so the statement has to be true.
         """
         cfg = self.cfg
         _require_gpu(weights, "weights")
@@ -265,7 +276,12 @@ class HipAllToAll:
         elif tuple(out.shape) != (rows, N) or out.dtype != cfg.out_dtype or not out.is_contiguous():
             raise ValueError("out must be out_dtype[rows, N], contiguous")
         common = (_ptr(d.offsets), _ptr(out), d.num_rows, E, H, N, d.max_recv, _elem(cfg.out_dtype), _stream())
-        if quant:
+        if scales_pow2:
+            if not (quant and fp8):
+                raise ValueError("scales_pow2 needs fp8 dispatched rows and block-quantised weights")
+            _lib.check(self.lib.moe_a2a_expert_gemm_mx8(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(weights),
+                                                        _ptr(w_scale), *common), "moe_a2a_expert_gemm_mx8")
+        elif quant:
             _lib.check(self.lib.moe_a2a_expert_gemm_q8(_ptr(d.disp_x), _ptr(d.disp_scale) if fp8 else None,
                                                        _ptr(weights), _ptr(w_scale), *common),
                        "moe_a2a_expert_gemm_q8")
@@ -323,7 +339,7 @@ class HipAllToAll:
         T, H = x.shape
         fuse_route = 2 if self.fuse_route == "always" else int(bool(self.fuse_route))
         return (_ptr(x), _ptr(indices), _ptr(weights), _ptr(rank_start), self.rank, T, cfg.experts_per_token,
-                cfg.num_experts, self.world_size, H, self.max_recv if self.padded else 0, _elem(cfg.in_dtype), _elem(cfg.out_dtype), int(self.fp8_dispatch),
+                cfg.num_experts, self.world_size, H, self.max_recv if self.padded else 0, _elem(cfg.in_dtype), _elem(cfg.out_dtype), 2 if self.fp8_dispatch == "pow2" else int(self.fp8_dispatch),
                 self.stub_kind, self.combine_mode, fuse_route, int(self.fuse_stub), _ptr(b["counts"]),
                 _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]), _ptr(b["meta"]),
                 _ptr(b["status"]), _ptr(b["disp_x"]), _ptr(b["disp_scale"]), _ptr(b["expert_y"]), _ptr(b["out"]),

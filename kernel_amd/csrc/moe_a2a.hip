@@ -58,12 +58,13 @@ enum KernelId {
   KID_EXPERT_GEMM_WIDE,
   KID_EXPERT_GEMM_SKINNY,
   KID_EXPERT_GEMM_F8,
+  KID_EXPERT_GEMM_MX,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
-    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8"};
+    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -796,14 +797,15 @@ __global__ __launch_bounds__(kTileThreads) void route_dispatch_tile_kernel(Route
 }
 
 // fp8 dispatch.  8 lanes own one 128-column block (16 elements each): block amax by three
-// xor-shuffles, scale = amax/448, q = e4m3(x/scale) with the hardware conversion (RNE).
+// xor-shuffles, scale = amax/448 (pow2: rounded up to a power of two, the scale format of the
+// matrix instruction's block exponents), q = e4m3(x/scale) with the hardware conversion (RNE).
 // Geometry is in lanes of 16 input elements: nvec = 8 * nblk, per a multiple of 8.
 template <class E, int STREAM>
 __global__ __launch_bounds__(kRowMaxThreads) void dispatch_fp8_kernel(const uint4* __restrict__ x,
                                                                        const int32_t* __restrict__ slot_of_entry,
                                                                        uint4* __restrict__ disp_q,
                                                                        float* __restrict__ disp_scale, int K,
-                                                                       int nblk, int per, int nsplit) {
+                                                                       int nblk, int per, int nsplit, int pow2) {
   const RowCut r = row_cut(nblk * 8, per, nsplit);
   float f[16];
   if (r.active) {
@@ -826,7 +828,12 @@ __global__ __launch_bounds__(kRowMaxThreads) void dispatch_fp8_kernel(const uint
   amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
   amax = fmaxf(amax, __shfl_xor(amax, 4, kWave));
   if (!r.active) return;
-  const float scale = amax == 0.f ? 1.f : amax / 448.f;
+  float scale = amax == 0.f ? 1.f : amax / 448.f;
+  if (pow2) {  // the next power of two at or above amax / 448, within the normal range
+    const uint32_t u = __float_as_uint(scale);
+    const uint32_t e = min(max((u >> 23) + ((u & 0x7fffffu) != 0 ? 1u : 0u), 1u), 254u);
+    scale = __uint_as_float(e << 23);
+  }
   uint32_t q[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -1292,6 +1299,7 @@ __global__ __launch_bounds__(kGemmThreads) void expert_gemm_kernel(const uint4* 
 constexpr int kWideM = 256, kWideN = 256, kWideK = 64, kWideLd = kWideK + 8, kWideThreads = 256;
 constexpr size_t kWideLdsBytes = 2 * (size_t)(kWideM + kWideN) * kWideLd * sizeof(uint16_t);
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
 
 template <class E>
 __device__ __forceinline__ f32x16_t mfma_32x32x16_v(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c);
@@ -1643,7 +1651,7 @@ __global__ __launch_bounds__(kSkinnyThreads, 3) void expert_gemm_skinny_q_kernel
 // Main loop and epilogue of one wide tile.  Each wave owns WMI x WNJ accumulator blocks of 32 x 32
 // at (wm, wn); AROWS rows of the A operand are staged per slab (256, or 128 when the tile holds
 // no more rows than that), always 256 rows of B.
-template <class E, int WMI, int WNJ, int AROWS, bool AFP8, bool BFP8>
+template <class E, int WMI, int WNJ, int AROWS, bool AFP8, bool BFP8, bool MX = false>
 __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const float* __restrict__ xs,
                                           const u32x4_t* __restrict__ wb, const float* __restrict__ wsc,
                                           uint16_t* __restrict__ y_tile, uint16_t* s_wide, int rows, int ncols,
@@ -1659,6 +1667,12 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
   // per tile: wsc[0..] and wsc[Kd/128..]); a vector is turned into two 16-bit vectors,
   // E(f32(q) * scale), on its way into LDS, so the LDS image and the number of LDS stores per
   // thread are those of the 16-bit case.
+  // MX: both operands are fp8 bytes that go to the fp8 matrix instruction as they are, with scales
+  // that are powers of two and ride along as the instruction's block exponents.  The caller passes
+  // Kd = bytes per row / 2, so a row looks like a 16-bit row of half the length and everything on
+  // the way into LDS is the 16-bit case; a slab of 64 such elements is one 128-wide scale block.
+  // xs = the tile's first row of x_scale, wsc = the scales of this wave's 128-column block.
+  static_assert(!MX || (!AFP8 && !BFP8), "MX operands are copied, not decoded");
   constexpr int VPR = BK / 8;
   constexpr int AVPR = AFP8 ? BK / 16 : VPR, BVPR = BFP8 ? BK / 16 : VPR;  // global vectors per row and slab
   constexpr int NA = AROWS * AVPR / NT, NB = TN * BVPR / NT;               // ... per thread
@@ -1680,6 +1694,13 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
   u32x4_t ra[NA], rb[NB];
   float rs[NS > 0 ? NS : 1];
   float rsb[2] = {1.f, 1.f};  // weight scales of the tile's two column blocks for the slab in flight
+  // MX: scale of each of the lane's WMI rows (row lane % 32 of every 32-row block) for the slab in flight
+  int mx_off[MX ? WMI : 1];  // a tile's scales span at most 256 rows x Kd / 64 floats: an int offset
+  float mx_rsa[MX ? WMI : 1];
+  if (MX) {
+#pragma unroll
+    for (int i = 0; i < WMI; ++i) mx_off[i] = min(wm + i * 32 + (lane & 31), rows - 1) * (Kd / 64);
+  }
   const int sb1 = ncols > 128 ? Kd / 128 : 0;  // a tile of one column block reads its scale twice
   const int st_off_a = (tid / AVPR) * LD + (tid % AVPR) * (AFP8 ? 16 : 8);
   const int st_off_b = (tid / BVPR) * LD + (tid % BVPR) * (BFP8 ? 16 : 8);
@@ -1691,6 +1712,10 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
     if (BFP8) {                                                                                  \
       rsb[0] = wsc[(K0) >> 7];                                                                   \
       rsb[1] = wsc[sb1 + ((K0) >> 7)];                                                           \
+    }                                                                                            \
+    if (MX) {                                                                                    \
+      _Pragma("unroll") for (int i = 0; i < WMI; ++i) mx_rsa[i] = xs[mx_off[i] + ((K0) >> 6)];   \
+      rsb[0] = wsc[(K0) >> 6];                                                                   \
     }                                                                                            \
   }
 #define WIDE_STASH(BUF)                                                                                        \
@@ -1782,6 +1807,86 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
 
   // The prefetches past the last slab re-read the last slab (clamped k) and land in a buffer
   // nobody reads: the loop body stays free of branches.
+  if constexpr (MX) {
+    // One slab = two steps of the fp8 instruction; a lane's operand is 32 bytes, read as the two
+    // 16-byte fragments the 16-bit loop reads for a pair of its steps (the same bytes for both
+    // operands, so the order in which the instruction walks K inside a step does not matter, and
+    // all its blocks of 32 carry the same exponent here).  Step 0 multiplies while step 1's
+    // fragments are read; step 1's first half while the next slab goes into the other buffer and
+    // the slab after that is requested; its second half while the next slab's first fragments
+    // are read.
+    u32x4_t f2a[WMI], f2b[WNJ], f3a[WMI], f3b[WNJ];
+    int sa_cur[WMI], sa_nxt[WMI], sb_cur, sb_nxt;
+#define MX_OPERAND(LO, HI) \
+  i32x8_t{(int)LO[0], (int)LO[1], (int)LO[2], (int)LO[3], (int)HI[0], (int)HI[1], (int)HI[2], (int)HI[3]}
+#define MX_MMA(LOA, HIA, LOB, HIB, I0, I1)                                                             \
+  {                                                                                                    \
+    _Pragma("unroll") for (int i = (I0); i < (I1); ++i)                                                \
+    _Pragma("unroll") for (int j = 0; j < WNJ; ++j)                                                    \
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                   \
+            MX_OPERAND(LOA[i], HIA[i]), MX_OPERAND(LOB[j], HIB[j]), acc[i][j], 0, 0, 0, sa_cur[i], 0, sb_cur); \
+  }
+#define MX_TAKE_SCALES() /* exponent fields of the slab that has just arrived */                       \
+  {                                                                                                    \
+    _Pragma("unroll") for (int i = 0; i < WMI; ++i) sa_nxt[i] = (__float_as_int(mx_rsa[i]) >> 23) & 0xff; \
+    sb_nxt = (__float_as_int(rsb[0]) >> 23) & 0xff;                                                    \
+  }
+    constexpr int HM = WMI / 2 * WNJ;  // MFMAs of half a step
+    WIDE_FETCH(0);
+    WIDE_STASH(0);
+    MX_TAKE_SCALES();
+#pragma unroll
+    for (int i = 0; i < WMI; ++i) sa_cur[i] = sa_nxt[i];
+    sb_cur = sb_nxt;
+    WIDE_FETCH(min(BK, Kd - BK));
+    __syncthreads();
+    WIDE_FRAGS(f0a, f0b, 0, 0);
+    WIDE_FRAGS(f1a, f1b, 0, 16);
+    int buf = 0;
+    for (int k0 = 0; k0 < Kd; k0 += BK, buf ^= 1) {
+      WIDE_FRAGS(f2a, f2b, buf, 32);
+      WIDE_FRAGS(f3a, f3b, buf, 48);
+      MX_MMA(f0a, f1a, f0b, f1b, 0, WMI);
+#pragma unroll
+      for (int s_ = 0; s_ < 2 * HM; ++s_) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (2 * RD + 2 * HM - 1) / (2 * HM), 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();  // every wave has left the previous slab: the other buffer is free
+      WIDE_STASH(buf ^ 1);
+      MX_TAKE_SCALES();
+      WIDE_FETCH(min(k0 + 2 * BK, Kd - BK));
+      MX_MMA(f2a, f3a, f2b, f3b, 0, WMI / 2);
+#pragma unroll
+      for (int s_ = 0; s_ < HM / 2; ++s_) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, (ST + HM / 2 - 1) / (HM / 2), 0);
+      }
+#pragma unroll
+      for (int s_ = 0; s_ < HM - HM / 2; ++s_) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, (ST + WMI + 1 + HM - HM / 2 - 1) / (HM - HM / 2), 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();  // the other buffer is complete
+      WIDE_FRAGS(f0a, f0b, buf ^ 1, 0);
+      WIDE_FRAGS(f1a, f1b, buf ^ 1, 16);
+      MX_MMA(f2a, f3a, f2b, f3b, WMI / 2, WMI);
+#pragma unroll
+      for (int s_ = 0; s_ < HM; ++s_) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (2 * RD + HM - 1) / HM, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < WMI; ++i) sa_cur[i] = sa_nxt[i];
+      sb_cur = sb_nxt;
+    }
+#undef MX_OPERAND
+#undef MX_MMA
+#undef MX_TAKE_SCALES
+  } else {
   WIDE_FETCH(0);
   WIDE_STASH(0);
   WIDE_FETCH(min(BK, Kd - BK));
@@ -1806,6 +1911,7 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
     WIDE_MMA(f1a, f1b);
     WIDE_MIX_READS();
   }
+  }
 #undef WIDE_FETCH
 #undef WIDE_STASH
 #undef WIDE_FRAGS
@@ -1826,7 +1932,9 @@ __device__ __forceinline__ void wide_tile(const u32x4_t* __restrict__ xa, const 
       }
 }
 
-template <class E, bool AFP8, bool BFP8>
+// MX: both operands fp8 with power-of-two scales, multiplied by the fp8 instruction with the
+// scales as its block exponents (see wide_tile).
+template <class E, bool AFP8, bool BFP8, bool MX = false>
 __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const uint4* __restrict__ x,
                                                                          const float* __restrict__ x_scale,
                                                                          const uint4* __restrict__ w,
@@ -1871,20 +1979,34 @@ __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const ui
   const int n0 = tile_n * TN;
   const int ncols = min(TN, N - n0);
   const int kvec = Kd / 8;
-  // fp8 rows are Kd bytes (Kd / 16 vectors) with Kd / 128 scales each
-  const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * (AFP8 ? Kd / 16 : kvec);
-  const float* xs = AFP8 ? x_scale + row0 * (Kd / 128) : nullptr;
-  const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * (BFP8 ? Kd / 16 : kvec);
-  // block-quantised weights: N % 128 == 0, the tile's first column block is n0 / 128
-  const float* wsc = BFP8 ? w_scale + ((size_t)e * (N / 128) + n0 / 128) * (Kd / 128) : nullptr;
   uint16_t* y_tile = y + row0 * (size_t)N + n0;
-  // A segment's last tile is often less than half full (23 % of the MFMAs of a 512-rows-per-expert
-  // ragged input would be spent on rows that do not exist): up to 128 rows the four waves stand
-  // side by side on 128 x 64 each, and only 128 rows of A are staged.
-  if (rows > 128)
-    wide_tile<E, 4, 4, 256, AFP8, BFP8>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd, N, (wave >> 1) * 128, (wave & 1) * 128);
-  else
-    wide_tile<E, 4, 2, 128, AFP8, BFP8>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd, N, 0, wave * 64);
+  if constexpr (MX) {
+    // rows and weight rows are Kd bytes (Kd / 16 vectors) with Kd / 128 scales; N % 128 == 0
+    const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * (Kd / 16);
+    const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * (Kd / 16);
+    const float* xs = x_scale + row0 * (Kd / 128);
+    const int wn = rows > 128 ? (wave & 1) * 128 : wave * 64;  // the wave's columns lie in one scale block
+    const int nblk = __builtin_amdgcn_readfirstlane(min(n0 + wn, N - 1) >> 7);
+    const float* wsc = w_scale + ((size_t)e * (N / 128) + nblk) * (Kd / 128);
+    if (rows > 128)
+      wide_tile<E, 4, 4, 256, false, false, true>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd / 2, N, (wave >> 1) * 128, wn);
+    else
+      wide_tile<E, 4, 2, 128, false, false, true>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd / 2, N, 0, wn);
+  } else {
+    // fp8 rows are Kd bytes (Kd / 16 vectors) with Kd / 128 scales each
+    const u32x4_t* xa = reinterpret_cast<const u32x4_t*>(x) + row0 * (AFP8 ? Kd / 16 : kvec);
+    const float* xs = AFP8 ? x_scale + row0 * (Kd / 128) : nullptr;
+    const u32x4_t* wb = reinterpret_cast<const u32x4_t*>(w) + ((size_t)e * N + n0) * (BFP8 ? Kd / 16 : kvec);
+    // block-quantised weights: N % 128 == 0, the tile's first column block is n0 / 128
+    const float* wsc = BFP8 ? w_scale + ((size_t)e * (N / 128) + n0 / 128) * (Kd / 128) : nullptr;
+    // A segment's last tile is often less than half full (23 % of the MFMAs of a 512-rows-per-expert
+    // ragged input would be spent on rows that do not exist): up to 128 rows the four waves stand
+    // side by side on 128 x 64 each, and only 128 rows of A are staged.
+    if (rows > 128)
+      wide_tile<E, 4, 4, 256, AFP8, BFP8>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd, N, (wave >> 1) * 128, (wave & 1) * 128);
+    else
+      wide_tile<E, 4, 2, 128, AFP8, BFP8>(xa, xs, wb, wsc, y_tile, s_wide, rows, ncols, Kd, N, 0, wave * 64);
+  }
 }
 
 // Both operands quantised: rows as the fp8 dispatch writes them (e4m3fn bytes + one f32 scale per
@@ -1904,7 +2026,6 @@ __global__ __launch_bounds__(kWideThreads) void expert_gemm_wide_kernel(const ui
 // belongs to the same row of x, and the fold needs one scale per lane and row block.
 constexpr int kF8M = 128, kF8K = 128, kF8Ld = kF8K + 16;
 constexpr int kXcds = 8;  // accelerator dies of an MI355X; workgroup b runs on die b % 8
-typedef int i32x8_t __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ f32x16_t mfma_32x32x64_fp8(const i32x8_t& a, const i32x8_t& b, const f32x16_t& c) {
   // formats 0 / 0 = e4m3 for both operands; the block exponents of the scaled form are 127 = 2^0
@@ -2394,8 +2515,10 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
 }
 
 int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry, uint8_t* disp_q,
-                         float* disp_scale, int T, int K, int H, moe_a2a_stream_t stream_) {
+                         float* disp_scale, int T, int K, int H, int scale_mode, moe_a2a_stream_t stream_) {
   if (x_type != MOE_A2A_F16 && x_type != MOE_A2A_BF16) return MOE_A2A_E_DTYPE;
+  if (scale_mode != MOE_A2A_FP8_SCALE_F32 && scale_mode != MOE_A2A_FP8_SCALE_POW2) return MOE_A2A_E_DTYPE;
+  const int pow2 = scale_mode == MOE_A2A_FP8_SCALE_POW2;
   if (int rc = check_rows(x, disp_q, T, K, H, MOE_A2A_FP8_BLOCK)) return rc;
   if (T == 0) return 0;
   if (!slot_of_entry || !disp_scale) return MOE_A2A_E_NULL;
@@ -2406,7 +2529,7 @@ int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry
   const bool st = streams(T, (long long)T * K, H, 2, 1);
 #define FP8_LAUNCH(EL, ST)                                                                                       \
   return launch(KID_DISPATCH_FP8, dispatch_fp8_kernel<EL, ST>, grid, block, 0, stream, (const uint4*)x, slot_of_entry, \
-                (uint4*)disp_q, disp_scale, K, nblk, g.per, g.nsplit)
+                (uint4*)disp_q, disp_scale, K, nblk, g.per, g.nsplit, pow2)
   if (x_type == MOE_A2A_BF16) {
     if (st) FP8_LAUNCH(Bf16, 1);
     FP8_LAUNCH(Bf16, 0);
@@ -2601,6 +2724,7 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                     int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
                     size_t workspace_bytes, moe_a2a_stream_t stream) {
   if (!known_type(in_type) || !known_type(out_type)) return MOE_A2A_E_DTYPE;
+  if (fp8_dispatch < 0 || fp8_dispatch > 2) return MOE_A2A_E_DTYPE;
   if (fp8_dispatch && !disp_scale) return MOE_A2A_E_NULL;
   if (!fuse_stub && T > 0 && !expert_y) return MOE_A2A_E_NULL;
   const bool fused = !fp8_dispatch && T > 0 &&
@@ -2614,6 +2738,8 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                                src_of_slot, meta, status, workspace, workspace_bytes, stream))
       return rc;
     if (int rc = fp8_dispatch ? moe_a2a_dispatch_fp8(x, in_type, slot_of_entry, (uint8_t*)disp, disp_scale, T, K, H,
+                                                     fp8_dispatch == 2 ? MOE_A2A_FP8_SCALE_POW2
+                                                                       : MOE_A2A_FP8_SCALE_F32,
                                                      stream)
                               : moe_a2a_dispatch(x, slot_of_entry, disp, T, K, H, stream))
       return rc;
@@ -2633,7 +2759,7 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
 // block-quantised weights.
 static int launch_gemm_wide(const void* x, const float* x_scale, const void* weights, const float* w_scale,
                             const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
-                            hipStream_t stream) {
+                            hipStream_t stream, bool mx = false) {
   const int ntile_n = ceil_div(N, kWideN);
   const long long mtiles = (long long)R / kWideM + E;  // every expert may end with a partly filled tile
   if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
@@ -2645,7 +2771,9 @@ static int launch_gemm_wide(const void* x, const float* x_scale, const void* wei
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= kMaxDevices) return MOE_A2A_E_STATE;
   if (!lds_raised[dev].load(std::memory_order_acquire)) {
-    const void* kernels[8] = {(const void*)expert_gemm_wide_kernel<Bf16, false, false>,
+    const void* kernels[10] = {(const void*)expert_gemm_wide_kernel<Bf16, false, false, true>,
+                              (const void*)expert_gemm_wide_kernel<F16, false, false, true>,
+                              (const void*)expert_gemm_wide_kernel<Bf16, false, false>,
                               (const void*)expert_gemm_wide_kernel<F16, false, false>,
                               (const void*)expert_gemm_wide_kernel<Bf16, true, false>,
                               (const void*)expert_gemm_wide_kernel<F16, true, false>,
@@ -2665,6 +2793,10 @@ static int launch_gemm_wide(const void* x, const float* x_scale, const void* wei
                 max_recv, ntile_n)
 #define CALL_WIDE_E(ET)                  \
   {                                      \
+    if (mx)                                                                                                    \
+      return launch(KID_EXPERT_GEMM_MX, expert_gemm_wide_kernel<ET, false, false, true>, grid, block,          \
+                    kWideLdsBytes, stream, (const uint4*)x, x_scale, (const uint4*)weights, w_scale, offsets,  \
+                    (uint16_t*)y, E, Kd, N, max_recv, ntile_n);                                                \
     if (x_scale && w_scale) CALL_WIDE(ET, true, true);  \
     if (x_scale) CALL_WIDE(ET, true, false);            \
     if (w_scale) CALL_WIDE(ET, false, true);            \
@@ -2791,6 +2923,28 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
   if (x_scale) CALL_SKQ(F16, true);
   CALL_SKQ(F16, false);
 #undef CALL_SKQ
+}
+
+int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w_q, const float* w_scale,
+                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
+                            moe_a2a_stream_t stream_) {
+  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
+  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 ||
+      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0)
+    return MOE_A2A_E_SHAPE;
+  if (R == 0) return 0;
+  if (!x_q || !x_scale || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
+  if (!aligned16(x_q) || !aligned16(w_q) || !aligned16(y)) return MOE_A2A_E_ALIGN;
+  // The 256 x 256 tiles pay off on long segments (measured at 512 rows per expert, 4096 -> 7168:
+  // 3109 us against 3420 us for the 128 x 128 kernel that folds the scales on the vector units; at
+  // 128 rows per expert 1316 against 1140 us); shorter ones go to moe_a2a_expert_gemm_q8, for which
+  // powers of two are f32 scales like any other.  MOE_A2A_GEMM_TILE=256 forces the tiles.
+  bool tiles = (long long)R >= 256ll * E;
+  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) tiles = atoi(forced) == 256;
+  if (!tiles)
+    return moe_a2a_expert_gemm_q8(x_q, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream_);
+  return launch_gemm_wide(x_q, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type,
+                          (hipStream_t)stream_, true);
 }
 
 int moe_a2a_timer_begin(int capacity) {

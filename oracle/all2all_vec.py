@@ -87,21 +87,32 @@ def dispatch(x: torch.Tensor, src_of_slot: torch.Tensor, K: int) -> torch.Tensor
     return x.index_select(0, (src_of_slot.to(torch.int64) // K))
 
 
-def quantize_fp8(x: torch.Tensor):
-    """Per-row, per-128-column e4m3fn quantisation; returns (q as uint8 bits, scale f32)."""
+def pow2_at_or_above(scale: torch.Tensor) -> torch.Tensor:
+    """The next power of two at or above a positive f32 (exponent field clamped to 1..254): the
+    power-of-two scale mode.  Done on the bits: exponent field + 1 when the mantissa is not zero."""
+    u = scale.contiguous().view(torch.int32)
+    e = (u >> 23) + ((u & 0x7FFFFF) != 0).to(torch.int32)
+    return (e.clamp(1, 254) << 23).view(torch.float32)
+
+
+def quantize_fp8(x: torch.Tensor, pow2: bool = False):
+    """Per-row, per-128-column e4m3fn quantisation; returns (q as uint8 bits, scale f32).
+    ``pow2``: the scale is ``amax / 448`` rounded up to a power of two."""
     T, H = x.shape
     assert H % FP8_BLOCK == 0
     xf = x.to(torch.float32).view(T, H // FP8_BLOCK, FP8_BLOCK)
     amax = xf.abs().amax(dim=-1)
     scale = amax / FP8_MAX
     scale = torch.where(amax == 0, torch.ones_like(scale), scale)
+    if pow2:
+        scale = pow2_at_or_above(scale)
     q = (xf / scale.unsqueeze(-1)).to(torch.float8_e4m3fn)
     return q.view(T, H).view(torch.uint8), scale
 
 
-def dispatch_fp8(x: torch.Tensor, src_of_slot: torch.Tensor, K: int):
+def dispatch_fp8(x: torch.Tensor, src_of_slot: torch.Tensor, K: int, pow2: bool = False):
     """Quantise each token row once, then copy rows and scales to their slots."""
-    q, scale = quantize_fp8(x)
+    q, scale = quantize_fp8(x, pow2)
     tok = src_of_slot.to(torch.int64) // K
     return q.index_select(0, tok), scale.index_select(0, tok)
 
@@ -156,15 +167,18 @@ def expert_gemm_fp8(q_bits: torch.Tensor, scale: torch.Tensor, offsets: torch.Te
     return expert_gemm(dequantize_fp8(q_bits, scale).to(weights.dtype), offsets, weights, out_dtype)
 
 
-def quantize_weights_fp8(weights: torch.Tensor):
+def quantize_weights_fp8(weights: torch.Tensor, pow2: bool = False):
     """Expert weights ``[E, N, Kd]`` -> e4m3fn bits and one f32 scale per 128 x 128 block
-    (``scale = amax / 448``, 1 for an all-zero block): the block format of DeepSeek-V3 checkpoints.
-    Test-side helper: the library only consumes weights in this format."""
+    (``scale = amax / 448``, 1 for an all-zero block; ``pow2``: rounded up to a power of two): the
+    block format of DeepSeek-V3 checkpoints.  Test-side helper: the library only consumes weights
+    in this format."""
     E, N, Kd = weights.shape
     assert N % FP8_BLOCK == 0 and Kd % FP8_BLOCK == 0
     wf = weights.to(torch.float32).view(E, N // FP8_BLOCK, FP8_BLOCK, Kd // FP8_BLOCK, FP8_BLOCK)
     amax = wf.abs().amax(dim=(2, 4))
     scale = torch.where(amax == 0, torch.ones_like(amax), amax / FP8_MAX)
+    if pow2:
+        scale = pow2_at_or_above(scale)
     q = (wf / scale[:, :, None, :, None]).to(torch.float8_e4m3fn)
     return q.view(E, N, Kd).view(torch.uint8), scale
 
@@ -228,7 +242,8 @@ def combine_f32(expert_y: torch.Tensor, weights: torch.Tensor, slot_of_entry: to
     return acc.to(out_dtype)
 
 
-def run_world(cfg, world: Sequence, stub_kind: int = 0, fp8: bool = False, combine_mode: int = 0):
+def run_world(cfg, world: Sequence, stub_kind: int = 0, fp8: bool = False, combine_mode: int = 0,
+              pow2: bool = False):
     """Whole path for an emulated world; returns every intermediate plus ``y[T,H]``."""
     x, idx, w, starts = concat_world(world)
     W = len(world)
@@ -236,7 +251,7 @@ def run_world(cfg, world: Sequence, stub_kind: int = 0, fp8: bool = False, combi
     r = route(idx, starts, cfg.num_experts)
     out = dict(r)
     if fp8:
-        q, sc = dispatch_fp8(x, r["src_of_slot"], K)
+        q, sc = dispatch_fp8(x, r["src_of_slot"], K, pow2)
         out.update(disp_x=q, disp_scale=sc)
         ey = stub(q, r["meta"], stub_kind, cfg.num_experts, W, cfg.out_dtype, scale=sc)
     else:

@@ -92,9 +92,10 @@ def test_row_functions_reject_bad_arguments(lib):
     assert lib.moe_a2a_dispatch(A + 4, A, A, 4, 2, 64, None) == E_ALIGN
     assert lib.moe_a2a_dispatch(A, None, A, 4, 2, 64, None) == E_NULL
     assert lib.moe_a2a_dispatch(A, A, A, 0, 2, 64, None) == 0  # nothing to do, nothing launched
-    assert lib.moe_a2a_dispatch_fp8(A, 7, A, A, A, 4, 2, 128, None) == E_DTYPE
-    assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, A, 4, 2, 64, None) == E_SHAPE  # H % 128
-    assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, None, 4, 2, 128, None) == E_NULL
+    assert lib.moe_a2a_dispatch_fp8(A, 7, A, A, A, 4, 2, 128, 0, None) == E_DTYPE
+    assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, A, 4, 2, 128, 2, None) == E_DTYPE  # scale mode
+    assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, A, 4, 2, 64, 0, None) == E_SHAPE  # H % 128
+    assert lib.moe_a2a_dispatch_fp8(A, _lib.BF16, A, A, None, 4, 2, 128, _lib.FP8_SCALE_POW2, None) == E_NULL
     assert lib.moe_a2a_stub(A, None, A, None, 5, _lib.BF16, 0, 8, 2, A, 8, 64, None) == E_DTYPE
     assert lib.moe_a2a_stub(A, None, A, None, _lib.BF16, _lib.BF16, 9, 8, 2, A, 8, 64, None) == E_DTYPE
     assert lib.moe_a2a_stub(A, None, A, None, _lib.BF16, _lib.BF16, 0, 9, 2, A, 8, 64, None) == E_SHAPE
@@ -136,6 +137,17 @@ def test_expert_gemm_rejects_bad_arguments(lib):
     assert gemmq(ws=None) == E_NULL
     assert gemmq(R=0) == 0
     assert gemmq(y=A + 4) == E_ALIGN
+
+    def gemmx(x=A, xs=A, w=A, ws=A, off=A, y=A, R=64, E=8, Kd=128, N=128, max_recv=0, elem=_lib.BF16):
+        return lib.moe_a2a_expert_gemm_mx8(x, xs, w, ws, off, y, R, E, Kd, N, max_recv, elem, None)
+
+    assert gemmx(elem=5) == E_DTYPE
+    assert gemmx(N=192) == E_SHAPE
+    assert gemmx(Kd=64) == E_SHAPE
+    assert gemmx(xs=None) == E_NULL  # the rows are fp8: their scales are required
+    assert gemmx(ws=None) == E_NULL
+    assert gemmx(R=0) == 0
+    assert gemmx(w=A + 8) == E_ALIGN
     assert gemm(Kd=72) == E_SHAPE    # hidden size in slabs of 64
     assert gemm8(Kd=192) == E_SHAPE  # fp8 rows carry one scale per 128 columns
     assert gemm8(sc=None) == E_NULL

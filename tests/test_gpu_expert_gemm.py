@@ -196,6 +196,39 @@ def test_expert_gemm_block_quantised_weights(gpu_device, monkeypatch, E, K, T, H
     close(y[rows], want[o["slot_of_entry"].long()])
 
 
+@pytest.mark.parametrize("E,K,T,H,N,W,zipf", [
+    (8, 2, 40, 128, 128, 1, False),      # 10 rows per expert: half tiles, one 128-column block
+    (4, 2, 300, 256, 256, 1, False),     # 150 rows per expert: half tiles
+    (16, 4, 300, 384, 384, 4, True),     # skewed: empty experts, long segments, a 128-column tail tile
+    (8, 2, 1200, 256, 512, 2, False),    # 300 rows per expert
+    (3, 1, 1000, 1024, 256, 1, False),   # 333 rows per expert, eight K blocks
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
+def test_expert_gemm_power_of_two_scales(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, padded):
+    """fp8 rows and fp8 weights whose scales are powers of two, multiplied by the fp8 matrix
+    instruction with the scales as its block exponents, against the f32 matmul of the
+    dequantised operands; the fp8 x fp8 kernel with the fold on the vector units, which takes
+    any f32 scale, has to agree with it to f32 summation order."""
+    monkeypatch.setenv("MOE_A2A_GEMM_TILE", "256")  # the tiles at every segment length
+    cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=7 * E + T, zipf=zipf)
+    wq, ws = V.quantize_weights_fp8(weights, pow2=True)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, fp8_dispatch="pow2", padded=padded, max_recv=T if padded else None)
+    d = ata.dispatch(x, idx, rs)
+    y = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device), scales_pow2=True)
+    monkeypatch.delenv("MOE_A2A_GEMM_TILE")
+    y_auto = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device), scales_pow2=True)  # library's choice
+    y_fold = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device))
+    torch.cuda.synchronize()
+    o = V.run_world(cfg, world, fp8=True, pow2=True)
+    want = V.expert_gemm_q8(o["disp_x"], o["disp_scale"], wq, ws, o["offsets"], dtype, round_rows=False)
+    rows = d.slot_of_entry.long() if padded else o["slot_of_entry"].long().to(gpu_device)
+    close(y[rows], want[o["slot_of_entry"].long()])
+    close(y[rows], y_fold[rows].cpu())
+    close(y_auto[rows], want[o["slot_of_entry"].long()])
+
+
 def test_dispatch_gemm_combine_end_to_end(gpu_device):
     """dispatch -> expert GEMM (H -> H) -> combine against the same chain on the CPU."""
     cfg, world, weights = make(32, 4, 512, 256, 256, 8, torch.bfloat16, seed=3)

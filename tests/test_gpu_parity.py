@@ -40,7 +40,7 @@ def assert_same(name, got, want):
 
 
 def compare(cfg, world, dev, stub_kind, combine_mode=0, fp8=False, fuse_route=True):
-    o = V.run_world(cfg, world, stub_kind=stub_kind, fp8=fp8, combine_mode=combine_mode)
+    o = V.run_world(cfg, world, stub_kind=stub_kind, fp8=bool(fp8), combine_mode=combine_mode, pow2=fp8 == "pow2")
     d, ey, y, y2 = run_hip(cfg, world, dev, stub_kind, combine_mode, fp8, fuse_route)
     assert int(d.status.item()) == 0
     assert_same("counts", d.counts, o["counts"])
@@ -167,6 +167,19 @@ def test_fp8_dispatch(gpu_device):
     wl = C.generate_workload("fp8_dispatch", tokens_scale=512 / 4096)
     compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, fp8=True)
     compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, fp8=True, combine_mode=C.COMBINE_F32)
+
+
+def test_fp8_dispatch_power_of_two_scales(gpu_device):
+    """The same path with scales rounded up to powers of two: bytes, scales and every later step
+    bit for bit, through the separate calls and through the one-call forward."""
+    wl = C.generate_workload("fp8_dispatch", tokens_scale=512 / 4096)
+    o, d = compare(wl.cfg, wl.world, gpu_device, wl.stub_kind, fp8="pow2")
+    assert bool((torch.frexp(d.disp_scale.cpu())[0] == 0.5).all())
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    ata = HipAllToAll(wl.cfg, 0, len(wl.world), stub_kind=wl.stub_kind, fp8_dispatch="pow2")
+    y = ata.forward(x, idx, w, rs)
+    torch.cuda.synchronize()
+    assert_same("y (forward)", y, o["y"])
 
 
 def test_duplicate_experts_and_ragged_world(gpu_device):

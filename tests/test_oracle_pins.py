@@ -200,6 +200,32 @@ def test_fp8_quantisation_definition_and_bound():
     assert float(sz.min()) == 1.0 and int(qz.max()) == 0
 
 
+def test_fp8_power_of_two_scales():
+    """Scale mode 2: the scale is the least power of two >= amax / 448 (so nothing saturates and at
+    most one bit of the e4m3 range is given up), the cast is the same, the error bound holds with
+    the block's own scale."""
+    wl = C.generate_workload("fp8_dispatch", tokens_scale=32 / 4096)
+    x = wl.world[0].x
+    q, scale = V.quantize_fp8(x, pow2=True)
+    T, H = x.shape
+    xf = x.float().view(T, H // 128, 128)
+    exact = xf.abs().amax(-1) / 448.0
+    mant, _ = torch.frexp(scale)
+    assert bool((mant == 0.5).all())                       # a power of two
+    assert bool((scale >= exact).all()) and bool((scale < 2 * exact).all())
+    ratio = (xf / scale.unsqueeze(-1)).numpy()
+    assert float(np.abs(ratio).max()) <= 448.0
+    assert np.array_equal(q.view(T, H // 128, 128).numpy(), encode_e4m3fn_nearest_even(ratio))
+    deq = V.dequantize_fp8(q, scale).view(T, H // 128, 128)
+    bound = torch.maximum(xf.abs() * 2.0 ** -4, scale.unsqueeze(-1) * 2.0 ** -10) * (1 + 1e-6)
+    assert bool(((deq - xf).abs() <= bound).all())
+    # closed cases of the rounding: powers of two stay, anything above moves up, the ends clamp
+    s = torch.tensor([1.0, 1.0 + 2.0 ** -23, 1.5, 2.0 ** -126, 1e-40, 3e38], dtype=torch.float32)
+    assert V.pow2_at_or_above(s).tolist() == [1.0, 2.0, 2.0, 2.0 ** -126, 2.0 ** -126, 2.0 ** 127]
+    wq, ws = V.quantize_weights_fp8(torch.randn(2, 128, 256), pow2=True)
+    assert bool((torch.frexp(ws)[0] == 0.5).all())
+
+
 def test_fp8_path_output_within_tolerance_of_bf16_path():
     wl = C.generate_workload("fp8_dispatch", tokens_scale=64 / 4096)
     a = V.run_world(wl.cfg, wl.world, stub_kind=1, fp8=True)["y"].float()
