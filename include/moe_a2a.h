@@ -242,14 +242,16 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
 /*
  * The same product for operands whose scales are all powers of two (rows from moe_a2a_dispatch_fp8
  * with MOE_A2A_FP8_SCALE_POW2, weights quantised with power-of-two block scales, the UE8M0 style
- * of newer DeepSeek checkpoints): on long segments (R >= 256 * E) the bytes of both operands go
- * to v_mfma_scale_f32_32x32x64_f8f6f4 and the exponent fields of the scales ride along as the
+ * of newer DeepSeek checkpoints): the bytes of both operands go to
+ * v_mfma_scale_f32_32x32x64_f8f6f4 and the exponent fields of the scales ride along as the
  * instruction's block exponents, so the products of all K blocks accumulate inside the matrix
- * cores (256 x 256 tiles, nothing is folded on the vector units).  y = sum over K blocks of
+ * cores (256 x 256 tiles, nothing is folded on the vector units; with Kd % 256 == 0 the operand
+ * slabs travel memory -> LDS directly, three slabs ahead).  y = sum over K blocks of
  * x_scale * w_scale * (q_x . q_w) in f32, one rounding to elem_type.  ONLY the exponent field of a
  * scale is used: a scale that is not a power of two is silently taken as the power of two below
- * it.  Shorter segments go through moe_a2a_expert_gemm_q8 (any f32 scale; MOE_A2A_GEMM_TILE=256
- * forces the tiles).  Arguments as for
+ * it.  Segments of at most 32 rows on average (a decode step), and other Kd on segments shorter
+ * than 256 rows, go through moe_a2a_expert_gemm_q8 (any f32 scale).  MOE_A2A_GEMM_TILE=256 forces
+ * the tiles, 32 / 128 the kernels of moe_a2a_expert_gemm_q8.  Arguments as for
  * moe_a2a_expert_gemm_q8 with x_scale required.  No counterpart in the reference.
  */
 int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w_q, const float* w_scale,

@@ -2224,6 +2224,228 @@ __global__ __launch_bounds__(2 * TN, TN == 128 ? 2 : 1) void expert_gemm_f8_kern
   }
 }
 
+// Power-of-two scales, slabs travelling memory -> LDS directly.  Ablation of the register-staged
+// loop above puts the cost where the slabs enter the CU: with the global loads taken out the same
+// loop runs 1.7 times faster, with the LDS stores out as well twice as fast, and its registers
+// leave no room to request a slab earlier.  Here a slab is 256 + 256 rows of 64 bytes (one step of
+// the fp8 instruction), global_load_lds (16 bytes per lane, 1 KB = 16 rows per wave instruction)
+// puts it into one of four 32 KB buffers, and slab s + 3 is requested while slab s is multiplied:
+// no staging registers, no LDS store instructions, three slabs in flight.  Rows of 64 bytes cannot
+// be padded, so the 16-byte chunk c of row r sits at chunk position c ^ ((r / 2) % 4): the reads
+// of eight consecutive rows then fall on disjoint banks.  The four buffers are separate arrays and
+// the loop is unrolled four times, so the compiler knows which buffer a read touches and does not
+// wait for the loads in flight to the others.  One barrier per slab, in the middle of its sixteen
+// MFMAs; the second eight hide the fragment reads of the next slab.
+constexpr int kMxdThreads = 256, kMxdSlab = (256 + 256) * 64;
+
+template <class E>
+__global__ __launch_bounds__(kMxdThreads) void expert_gemm_mxd_kernel(const uint4* __restrict__ x_q,
+                                                                      const float* __restrict__ x_scale,
+                                                                      const uint4* __restrict__ w_q,
+                                                                      const float* __restrict__ w_scale,
+                                                                      const int32_t* __restrict__ offsets,
+                                                                      uint16_t* __restrict__ y, int num_experts,
+                                                                      int Kd, int N, int max_recv, int ntile_n) {
+  constexpr int TM = 256, TN = 256, NT = kMxdThreads, ROWB = 64;
+  __shared__ __attribute__((aligned(1024))) uint8_t s_b0[kMxdSlab];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_b1[kMxdSlab];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_b2[kMxdSlab];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_b3[kMxdSlab];
+  __shared__ int s_pref[MOE_A2A_MAX_EXPERTS + 1];
+  __shared__ int s_tmp[NT / kWave + 1];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+
+  const int tile_n = blockIdx.x % ntile_n;
+  const int tile_m_global = blockIdx.x / ntile_n;
+  {
+    const int span = (num_experts + NT - 1) / NT;
+    const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    int total;
+    int run = block_exclusive_scan(sum, s_tmp, total);
+    for (int e = lo; e < hi; ++e) {
+      s_pref[e] = run;
+      run += (offsets[e + 1] - offsets[e] + TM - 1) / TM;
+    }
+    if (tid == 0) s_pref[num_experts] = total;
+    __syncthreads();
+    if (tile_m_global >= total) return;
+  }
+  int e_lo = 0, e_hi = num_experts;
+  while (e_hi - e_lo > 1) {
+    int mid = (e_lo + e_hi) >> 1;
+    if (s_pref[mid] <= tile_m_global) e_lo = mid; else e_hi = mid;
+  }
+  const int e = e_lo;
+  const int count = offsets[e + 1] - offsets[e];
+  const int m0 = (tile_m_global - s_pref[e]) * TM;
+  const size_t row0 = (size_t)(max_recv > 0 ? e * max_recv : offsets[e]) + m0;
+  const int rows = min(TM, count - m0);
+  const int n0 = tile_n * TN;
+  const int ncols = min(TN, N - n0);
+  const int kvec = Kd / 16, kblk = Kd / 128, nslab = Kd / ROWB;
+
+  // waves 0, 1 bring in the rows of x, waves 2, 3 the weight rows: eight instructions of sixteen
+  // rows per wave and slab; lane l fills row l / 4, chunk position l % 4 of its kilobyte
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  const u32x4_t* gsrc = wave < 2 ? reinterpret_cast<const u32x4_t*>(x_q) + row0 * kvec
+                                 : reinterpret_cast<const u32x4_t*>(w_q) + ((size_t)e * N + n0) * kvec;
+  const int limit = wave < 2 ? rows : ncols;  // rows past the end re-read the last one: never stored
+  int goff[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const int r = (wave & 1) * 128 + t * 16 + (lane >> 2);
+    goff[t] = min(r, limit - 1) * kvec + ((lane & 3) ^ ((r >> 1) & 3));
+  }
+  const int lds_wave = wave * 8 * 1024;  // x rows are the first 16 KB of a buffer, weight rows the second
+#define MXD_ISSUE(S, BUFP)                                                                                   \
+  {                                                                                                          \
+    const int s_ = min((S), nslab - 1); /* past the end: the last slab again, into a buffer nobody reads */  \
+    _Pragma("unroll") for (int t = 0; t < 8; ++t)                                                            \
+        __builtin_amdgcn_global_load_lds((gptr_t)(gsrc + goff[t] + s_ * 4), (lptr_t)(BUFP + lds_wave + t * 1024), \
+                                         16, 0, 0);                                                          \
+  }
+  const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+  // Scales: the exponent fields go to the instruction.  The row scales of a 128-wide block (two
+  // slabs) travel memory -> LDS as well, one float per row (a vector load into registers here
+  // would make the compiler wait for every load in flight whenever its value is used): wave w
+  // fetches rows 64 w .. 64 w + 63, two blocks ahead, into the array of the block's parity; a
+  // lane reads the four it needs (row lane % 32 of its wave's four 32-row blocks) one step before
+  // the block starts.  The weight scale is uniform over the wave: a scalar load.
+  __shared__ __attribute__((aligned(256))) float s_sc0[TM];
+  __shared__ __attribute__((aligned(256))) float s_sc1[TM];
+  const float* xs = x_scale + (row0 + min(wave * 64 + lane, rows - 1)) * kblk;
+  const float* wsc = w_scale + ((size_t)e * (N / 128) + __builtin_amdgcn_readfirstlane(min(n0 + wn, N - 1) >> 7)) * kblk;
+  int sa_cur[4], sa_nxt[4], sb_cur, sb_nxt;
+#define MXD_SCALES_ISSUE(KB, SCP) \
+  __builtin_amdgcn_global_load_lds((gptr_t)(xs + min((KB), kblk - 1)), (lptr_t)(SCP + wave * 64), 4, 0, 0);
+#define MXD_SCALES_READ(KB, SCP, SA, SB)                                                                     \
+  {                                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                            \
+        SA[i] = (__float_as_int(SCP[wm + i * 32 + (lane & 31)]) >> 23) & 0xff;                               \
+    SB = (__float_as_int(wsc[min((KB), kblk - 1)]) >> 23) & 0xff;                                            \
+  }
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+  // fragment of a lane: row lane % 32 of a block, chunks 2 h and 2 h + 1 of the four, h = lane / 32,
+  // at their swizzled positions ((row / 2) % 4 == (lane / 2) % 4: blocks start at multiples of 32)
+  const int sw = (lane >> 1) & 3;
+  const int p0 = (((lane >> 5) * 2) ^ sw) * 16, p1 = (((lane >> 5) * 2 + 1) ^ sw) * 16;
+  const int fr_a = (wm + (lane & 31)) * ROWB, fr_b = (TM + wn + (lane & 31)) * ROWB;
+  i32x8_t pa[4], pb[4], qa[4], qb[4];
+#define MXD_LOAD8(DST, PTR)                                                                                  \
+  {                                                                                                          \
+    const u32x4_t lo_ = *reinterpret_cast<const u32x4_t*>(&(PTR)[p0]);                                       \
+    const u32x4_t hi_ = *reinterpret_cast<const u32x4_t*>(&(PTR)[p1]);                                       \
+    DST = i32x8_t{(int)lo_[0], (int)lo_[1], (int)lo_[2], (int)lo_[3], (int)hi_[0], (int)hi_[1], (int)hi_[2], (int)hi_[3]}; \
+  }
+#define MXD_FRAGS(FA, FB, BUFP)                                                                              \
+  {                                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) MXD_LOAD8(FA[i], BUFP + fr_a + i * 32 * ROWB);             \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) MXD_LOAD8(FB[j], BUFP + fr_b + j * 32 * ROWB);             \
+  }
+#define MXD_MMA(FA, FB, I0, I1)                                                                              \
+  {                                                                                                          \
+    _Pragma("unroll") for (int i = (I0); i < (I1); ++i)                                                      \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                            \
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA[i], FB[j], acc[i][j], 0, 0, 0, sa_cur[i], 0, \
+                                                                    sb_cur);                                 \
+  }
+  // One slab: request slab S + 3 into DBUF (the buffer of slab S - 1, which every wave has left),
+  // multiply the first half of slab S from the fragments FA / FB, make sure slab S + 1 has landed
+  // for every wave (vmcnt(17): at most the 16 load instructions of slabs S + 2 and S + 3 and the
+  // one scale load between them are pending; then the barrier), read its fragments from RBUF into
+  // GA / GB in the shadow of the second half.  PRE and POST are the scale traffic of even steps.
+#define MXD_STEP(S, DBUF, RBUF, FA, FB, GA, GB, PRE, POST)                                                   \
+  {                                                                                                          \
+    PRE;                                                                                                     \
+    MXD_ISSUE((S) + 3, DBUF);                                                                                \
+    MXD_MMA(FA, FB, 0, 2);                                                                                   \
+    /* one load instruction behind each MFMA: a wave that waits for the address unit to take a load */      \
+    /* issues nothing else, and an MFMA in flight covers 64 clocks of that */                                \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                     \
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                     \
+    }                                                                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                       \
+    asm volatile("" ::: "memory");                                                                           \
+    __builtin_amdgcn_s_waitcnt(0x4F71); /* vmcnt(17) */                                                      \
+    __builtin_amdgcn_s_barrier();                                                                            \
+    asm volatile("" ::: "memory");                                                                           \
+    __builtin_amdgcn_sched_barrier(0);                                                                       \
+    MXD_FRAGS(GA, GB, RBUF);                                                                                 \
+    POST;                                                                                                    \
+    MXD_MMA(FA, FB, 2, 4);                                                                                   \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                     \
+      __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);                                                     \
+    }                                                                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                       \
+  }
+  MXD_SCALES_ISSUE(0, s_sc0);
+  MXD_SCALES_ISSUE(1, s_sc1);
+  MXD_ISSUE(0, s_b0);
+  MXD_ISSUE(1, s_b1);
+  MXD_ISSUE(2, s_b2);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): the scales of blocks 0 and 1 and slab 0 are in
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  MXD_SCALES_READ(0, s_sc0, sa_cur, sb_cur);
+  MXD_FRAGS(pa, pb, s_b0);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave has read the scales of block 0 ...
+  __builtin_amdgcn_s_barrier();        // ... and so has every other: the first step may overwrite them
+  asm volatile("" ::: "memory");
+  // A 128-wide scale block is two slabs.  On the first slab of block b the scales of block b + 2
+  // are requested (into the array block b used: every wave read it a barrier ago) and those of
+  // block b + 1 are read (they were requested two steps earlier and have landed with this step's
+  // wait); after its second slab they become current.  Kd is a multiple of 256 here, so the
+  // number of slabs is a multiple of four.
+#pragma clang loop unroll(disable)
+  for (int s = 0; s < nslab; s += 4) {
+    MXD_STEP(s, s_b3, s_b1, pa, pb, qa, qb, MXD_SCALES_ISSUE(s / 2 + 2, s_sc0),
+             MXD_SCALES_READ(s / 2 + 1, s_sc1, sa_nxt, sb_nxt));
+    MXD_STEP(s + 1, s_b0, s_b2, qa, qb, pa, pb, , );
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sa_cur[i] = sa_nxt[i];
+    sb_cur = sb_nxt;
+    MXD_STEP(s + 2, s_b1, s_b3, pa, pb, qa, qb, MXD_SCALES_ISSUE(s / 2 + 3, s_sc1),
+             MXD_SCALES_READ(s / 2 + 2, s_sc0, sa_nxt, sb_nxt));
+    MXD_STEP(s + 3, s_b2, s_b0, qa, qb, pa, pb, , );
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sa_cur[i] = sa_nxt[i];
+    sb_cur = sb_nxt;
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing may land after the LDS is given back
+#undef MXD_ISSUE
+#undef MXD_SCALES_ISSUE
+#undef MXD_SCALES_READ
+#undef MXD_FRAGS
+#undef MXD_LOAD8
+#undef MXD_MMA
+#undef MXD_STEP
+
+  uint16_t* y_tile = y + row0 * (size_t)N + n0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int r = wm + i * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
+        const int c = wn + j * 32 + (lane & 31);
+        if (r < rows && c < ncols) y_tile[r * (size_t)N + c] = (uint16_t)(E::pack(acc[i][j][q], 0.f) & 0xffffu);
+      }
+}
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -2935,14 +3157,40 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
   if (R == 0) return 0;
   if (!x_q || !x_scale || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
   if (!aligned16(x_q) || !aligned16(w_q) || !aligned16(y)) return MOE_A2A_E_ALIGN;
-  // The 256 x 256 tiles pay off on long segments (measured at 512 rows per expert, 4096 -> 7168:
-  // 3109 us against 3420 us for the 128 x 128 kernel that folds the scales on the vector units; at
-  // 128 rows per expert 1316 against 1140 us); shorter ones go to moe_a2a_expert_gemm_q8, for which
-  // powers of two are f32 scales like any other.  MOE_A2A_GEMM_TILE=256 forces the tiles.
-  bool tiles = (long long)R >= 256ll * E;
-  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) tiles = atoi(forced) == 256;
-  if (!tiles)
+  // A decode step (R <= 32 E) is bound by the weight bytes: moe_a2a_expert_gemm_q8 streams them, and
+  // powers of two are f32 scales like any other.  Otherwise 256 x 256 tiles with the scales as block
+  // exponents: slabs sent memory -> LDS directly when Kd is a multiple of 256 (measured against the
+  // kernel that folds f32 scales on the vector units: 1059 / 1140 us at 128 rows per expert,
+  // 7168 -> 2048; 815 / 923 us and 2533 / 3420 us at 512 rows per expert, 4096 -> 2048 and -> 7168),
+  // the register-staged loop for other Kd on long segments (3109 us in the last case), the folding
+  // kernel for what is left.  MOE_A2A_GEMM_TILE = 32 | 128 force the streaming / the folding kernel,
+  // 256 the tiles; MOE_A2A_MX_STAGED = 1 the register-staged loop.
+  enum { kStream, kFold, kTilesDirect, kTilesStaged } kernel;
+  const bool staged_only = Kd % 256 != 0 || (getenv("MOE_A2A_MX_STAGED") && atoi(getenv("MOE_A2A_MX_STAGED")) == 1);
+  if ((long long)R <= 32ll * E) kernel = kStream;
+  else if (!staged_only) kernel = kTilesDirect;
+  else kernel = (long long)R >= 256ll * E ? kTilesStaged : kFold;
+  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) {
+    const int tile = atoi(forced);
+    if (tile == 32) kernel = kStream;
+    if (tile == 128) kernel = kFold;
+    if (tile == 256) kernel = staged_only ? kTilesStaged : kTilesDirect;
+  }
+  if (kernel == kStream || kernel == kFold)  // the same environment variable picks between the two there
     return moe_a2a_expert_gemm_q8(x_q, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream_);
+  if (kernel == kTilesDirect) {
+    const int ntile_n = ceil_div(N, 256);
+    const long long mtiles = (long long)R / 256 + E;
+    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
+    dim3 grid((unsigned)(mtiles * ntile_n)), block(kMxdThreads);
+    if (elem_type == MOE_A2A_BF16)
+      return launch(KID_EXPERT_GEMM_MX, expert_gemm_mxd_kernel<Bf16>, grid, block, 0, (hipStream_t)stream_,
+                    (const uint4*)x_q, x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv,
+                    ntile_n);
+    return launch(KID_EXPERT_GEMM_MX, expert_gemm_mxd_kernel<F16>, grid, block, 0, (hipStream_t)stream_,
+                  (const uint4*)x_q, x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv,
+                  ntile_n);
+  }
   return launch_gemm_wide(x_q, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type,
                           (hipStream_t)stream_, true);
 }

@@ -202,15 +202,23 @@ def test_expert_gemm_block_quantised_weights(gpu_device, monkeypatch, E, K, T, H
     (16, 4, 300, 384, 384, 4, True),     # skewed: empty experts, long segments, a 128-column tail tile
     (8, 2, 1200, 256, 512, 2, False),    # 300 rows per expert
     (3, 1, 1000, 1024, 256, 1, False),   # 333 rows per expert, eight K blocks
+    (5, 2, 700, 768, 640, 1, True),      # twelve slabs of 64 bytes, a 128-column tail tile, ragged
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-def test_expert_gemm_power_of_two_scales(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, padded):
+@pytest.mark.parametrize("staged", [False, True], ids=["direct", "staged"])
+def test_expert_gemm_power_of_two_scales(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, padded, staged):
     """fp8 rows and fp8 weights whose scales are powers of two, multiplied by the fp8 matrix
     instruction with the scales as its block exponents, against the f32 matmul of the
     dequantised operands; the fp8 x fp8 kernel with the fold on the vector units, which takes
-    any f32 scale, has to agree with it to f32 summation order."""
+    any f32 scale, has to agree with it to f32 summation order.  Both forms of the tiled kernel:
+    slabs sent memory -> LDS directly (hidden sizes that are multiples of 256) and staged through
+    registers (every hidden size)."""
     monkeypatch.setenv("MOE_A2A_GEMM_TILE", "256")  # the tiles at every segment length
+    if staged:
+        monkeypatch.setenv("MOE_A2A_MX_STAGED", "1")
+    else:
+        monkeypatch.delenv("MOE_A2A_MX_STAGED", raising=False)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=7 * E + T, zipf=zipf)
     wq, ws = V.quantize_weights_fp8(weights, pow2=True)
     x, idx, w, rs = concat_world(world, gpu_device)
@@ -327,18 +335,20 @@ def test_random_shapes_every_expert_gemm_form(gpu_device, monkeypatch, seed):
     padded = pick([False, True])
     fp8_rows = pick([False, True])
     q8 = pick([False, True])
+    pow2 = pick([False, True]) and fp8_rows and q8  # scales as the matrix instruction's block exponents
     if seed % 2:
         monkeypatch.setenv("MOE_A2A_GEMM_TILE", pick(["32", "128", "256"]))
     else:
         monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=seed, zipf=zipf)
     x, idx, w, rs = concat_world(world, gpu_device)
-    ata = HipAllToAll(cfg, 0, W, fp8_dispatch=fp8_rows, padded=padded, max_recv=T if padded else None)
+    ata = HipAllToAll(cfg, 0, W, fp8_dispatch="pow2" if pow2 else fp8_rows, padded=padded,
+                      max_recv=T if padded else None)
     d = ata.dispatch(x, idx, rs)
-    o = V.run_world(cfg, world, fp8=fp8_rows)
+    o = V.run_world(cfg, world, fp8=fp8_rows, pow2=pow2)
     if q8:
-        wq, ws = V.quantize_weights_fp8(weights)
-        y = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device))
+        wq, ws = V.quantize_weights_fp8(weights, pow2=pow2)
+        y = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device), scales_pow2=pow2)
         # which of the q8 kernels ran decides whether fp8 rows were rounded to 16 bits first; both
         # readings of the rows differ by far less than the tolerance, so the unrounded one serves
         want = V.expert_gemm_q8(o["disp_x"], o["disp_scale"] if fp8_rows else None, wq, ws, o["offsets"], dtype,
