@@ -2234,8 +2234,8 @@ __global__ __launch_bounds__(2 * TN, TN == 128 ? 2 : 1) void expert_gemm_f8_kern
 // be padded, so the 16-byte chunk c of row r sits at chunk position c ^ ((r / 2) % 4): the reads
 // of eight consecutive rows then fall on disjoint banks.  The four buffers are separate arrays and
 // the loop is unrolled four times, so the compiler knows which buffer a read touches and does not
-// wait for the loads in flight to the others.  One barrier per slab, in the middle of its sixteen
-// MFMAs; the second eight hide the fragment reads of the next slab.
+// wait for the loads in flight to the others.  One barrier per slab, at its top; the sixteen MFMAs
+// hide the fragment reads of the next slab and the issue of the loads.
 constexpr int kMxdThreads = 256, kMxdSlab = (256 + 256) * 64;
 
 template <class E>
@@ -2358,34 +2358,35 @@ __global__ __launch_bounds__(kMxdThreads) void expert_gemm_mxd_kernel(const uint
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FA[i], FB[j], acc[i][j], 0, 0, 0, sa_cur[i], 0, \
                                                                     sb_cur);                                 \
   }
-  // One slab: request slab S + 3 into DBUF (the buffer of slab S - 1, which every wave has left),
-  // multiply the first half of slab S from the fragments FA / FB, make sure slab S + 1 has landed
-  // for every wave (vmcnt(17): at most the 16 load instructions of slabs S + 2 and S + 3 and the
-  // one scale load between them are pending; then the barrier), read its fragments from RBUF into
-  // GA / GB in the shadow of the second half.  PRE and POST are the scale traffic of even steps.
+  // One slab.  First make sure slab S + 1 has landed for every wave (vmcnt(8): at most the eight
+  // load instructions of slab S + 2 are pending; then the barrier -- which also says that every wave
+  // has left slab S - 1).  Then the sixteen MFMAs of slab S from the fragments FA / FB, and in their
+  // shadow: the request for slab S + 3 into DBUF (the buffer of slab S - 1), one load instruction
+  // behind each of the first eight MFMAs (a wave that waits for the address unit to take a load
+  // issues nothing else, and an MFMA in flight covers 64 clocks of that); the fragments of slab
+  // S + 1 from RBUF into GA / GB, one read behind each MFMA (spread over the whole slab the four
+  // waves ask the LDS for half of what it can deliver; packed behind eight MFMAs it was all of
+  // it).  PRE and POST are the scale traffic of even steps.
 #define MXD_STEP(S, DBUF, RBUF, FA, FB, GA, GB, PRE, POST)                                                   \
   {                                                                                                          \
-    PRE;                                                                                                     \
-    MXD_ISSUE((S) + 3, DBUF);                                                                                \
-    MXD_MMA(FA, FB, 0, 2);                                                                                   \
-    /* one load instruction behind each MFMA: a wave that waits for the address unit to take a load */      \
-    /* issues nothing else, and an MFMA in flight covers 64 clocks of that */                                \
-    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                       \
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                     \
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                     \
-    }                                                                                                        \
-    __builtin_amdgcn_sched_barrier(0);                                                                       \
     asm volatile("" ::: "memory");                                                                           \
-    __builtin_amdgcn_s_waitcnt(0x4F71); /* vmcnt(17) */                                                      \
+    __builtin_amdgcn_s_waitcnt(0x0F78); /* vmcnt(8) */                                                       \
     __builtin_amdgcn_s_barrier();                                                                            \
     asm volatile("" ::: "memory");                                                                           \
     __builtin_amdgcn_sched_barrier(0);                                                                       \
+    PRE;                                                                                                     \
+    MXD_ISSUE((S) + 3, DBUF);                                                                                \
     MXD_FRAGS(GA, GB, RBUF);                                                                                 \
     POST;                                                                                                    \
-    MXD_MMA(FA, FB, 2, 4);                                                                                   \
+    MXD_MMA(FA, FB, 0, 4);                                                                                   \
     _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                       \
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                     \
-      __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);                                                     \
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                     \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                     \
+    }                                                                                                        \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                                                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                     \
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                                                     \
     }                                                                                                        \
     __builtin_amdgcn_sched_barrier(0);                                                                       \
   }
