@@ -2255,8 +2255,14 @@ __global__ __launch_bounds__(kMxdThreads) void expert_gemm_mxd_kernel(const uint
   __shared__ int s_tmp[NT / kWave + 1];
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
 
-  const int tile_n = blockIdx.x % ntile_n;
-  const int tile_m_global = blockIdx.x / ntile_n;
+  // tile of this workgroup: every XCD (workgroup b runs on XCD b % 8, each with its own L2) takes a
+  // contiguous eighth of the m-tiles with all their n-tiles, so the rows of an m-tile are fetched
+  // into one L2 only (with the plain n-fastest map this launch reads its operands from memory
+  // nine times over)
+  const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+  const int tile_n = slot % ntile_n;
+  const int tile_m_local = slot / ntile_n;
+  int tile_m_global;
   {
     const int span = (num_experts + NT - 1) / NT;
     const int lo = min(tid * span, num_experts), hi = min(lo + span, num_experts);
@@ -2270,7 +2276,9 @@ __global__ __launch_bounds__(kMxdThreads) void expert_gemm_mxd_kernel(const uint
     }
     if (tid == 0) s_pref[num_experts] = total;
     __syncthreads();
-    if (tile_m_global >= total) return;
+    const int chunk = (total + kXcds - 1) / kXcds;
+    tile_m_global = xcd * chunk + tile_m_local;
+    if (tile_m_local >= chunk || tile_m_global >= total) return;  // the grid is sized for the worst case
   }
   int e_lo = 0, e_hi = num_experts;
   while (e_hi - e_lo > 1) {
@@ -3161,8 +3169,8 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
   // A decode step (R <= 32 E) is bound by the weight bytes: moe_a2a_expert_gemm_q8 streams them, and
   // powers of two are f32 scales like any other.  Otherwise 256 x 256 tiles with the scales as block
   // exponents: slabs sent memory -> LDS directly when Kd is a multiple of 256 (measured against the
-  // kernel that folds f32 scales on the vector units: 1059 / 1140 us at 128 rows per expert,
-  // 7168 -> 2048; 815 / 923 us and 2533 / 3420 us at 512 rows per expert, 4096 -> 2048 and -> 7168),
+  // kernel that folds f32 scales on the vector units: 1022 / 1140 us at 128 rows per expert,
+  // 7168 -> 2048; 735 / 923 us and 2592 / 3420 us at 512 rows per expert, 4096 -> 2048 and -> 7168),
   // the register-staged loop for other Kd on long segments (3109 us in the last case), the folding
   // kernel for what is left.  MOE_A2A_GEMM_TILE = 32 | 128 force the streaming / the folding kernel,
   // 256 the tiles; MOE_A2A_MX_STAGED = 1 the register-staged loop.
@@ -3181,7 +3189,8 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
     return moe_a2a_expert_gemm_q8(x_q, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream_);
   if (kernel == kTilesDirect) {
     const int ntile_n = ceil_div(N, 256);
-    const long long mtiles = (long long)R / 256 + E;
+    // worst case of m-tiles (every expert ends with a partly filled one), an eighth of them per XCD
+    const long long mtiles = ((long long)R / 256 + E + kXcds - 1) / kXcds * kXcds;
     if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
     dim3 grid((unsigned)(mtiles * ntile_n)), block(kMxdThreads);
     if (elem_type == MOE_A2A_BF16)
