@@ -835,8 +835,8 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
   // A decode step (R <= 32 E) is bound by the weight bytes: moe_a2a_expert_gemm_q8 streams them, and
   // powers of two are f32 scales like any other.  Otherwise 256 x 256 tiles with the scales as block
   // exponents: slabs sent memory -> LDS directly when Kd is a multiple of 256 (measured against the
-  // kernel that folds f32 scales on the vector units: 1022 / 1140 us at 128 rows per expert,
-  // 7168 -> 2048; 735 / 923 us and 2592 / 3420 us at 512 rows per expert, 4096 -> 2048 and -> 7168),
+  // kernel that folds f32 scales on the vector units: 951 / 1140 us at 128 rows per expert,
+  // 7168 -> 2048; 735 / 923 us and 2562 / 3420 us at 512 rows per expert, 4096 -> 2048 and -> 7168),
   // the register-staged loop for other Kd on long segments (3109 us in the last case), the folding
   // kernel for what is left.  MOE_A2A_GEMM_TILE = 32 | 128 force the streaming / the folding kernel,
   // 256 the tiles; MOE_A2A_MX_STAGED = 1 the register-staged loop.
