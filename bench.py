@@ -380,7 +380,7 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
     live = int((d.counts > 0).sum())
     # the kernel with both operands fp8 multiplies on the fp8 matrix instruction (dense peak 5.0 PFLOP/s)
     mfma_peak = FP8_MFMA_PEAK_TFLOPS if kernel in ("expert_gemm_f8", "expert_gemm_mx") else MFMA_PEAK_TFLOPS
-    if kernel in ("expert_gemm_f8", "expert_gemm_mx"):
+    if kernel in ("expert_gemm_f8", "expert_gemm_mx") or (fp8 and args.fp8_weights):
         out["dtype"] = "fp8"
     gemm_bytes = R * H * (1 + 4 / 128 if fp8 else 2) + live * N * H * (1 if args.fp8_weights else 2) + R * N * 2
     if gemm_bytes / (HBM_PEAK_GBPS * 1e3) > flops / (mfma_peak * 1e6):
