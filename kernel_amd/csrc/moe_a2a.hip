@@ -31,7 +31,8 @@ namespace {
 constexpr int kWave = 64;
 constexpr int kRouteThreads = 1024;
 constexpr int kRouteWaves = kRouteThreads / kWave;
-constexpr int kRouteTilesMaxRows = 16 * kRouteThreads;  // one-launch routing up to here
+constexpr int kRouteTilesMaxRows = 32 * kRouteThreads;  // one-launch routing up to here (8.7 against 10.2 us in two
+                                                        // launches at 32 K entries, 12.2 against 10.8 us at 64 K)
 constexpr int kRowMaxThreads = 512;
 constexpr int kFusedIdBits = 13;
 constexpr int kFusedMaxRows = 1 << kFusedIdBits;  // route_dispatch packs (expert, entry id) into one key

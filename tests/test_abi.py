@@ -50,6 +50,7 @@ def test_version_strings_and_queries(lib):
     assert {b"route_tiles", b"route_dispatch", b"dispatch_rows", b"dispatch_fp8", b"combine_rows"} <= names
     # small tables route in one launch and need only the minimum scratch
     assert lib.moe_a2a_workspace_bytes(256, 8, 256) == 256
+    assert lib.moe_a2a_workspace_bytes(4096, 8, 256) == 256
     assert lib.moe_a2a_workspace_bytes(16384, 4, 128) >= 64 * 128 * 4
     assert lib.moe_a2a_workspace_bytes(-1, 8, 256) == 0
     assert lib.moe_a2a_fused_max_rows() >= 2048

@@ -99,7 +99,7 @@ def test_named_workloads(gpu_device, name, scale, mode):
 
 
 def test_multi_workgroup_routing(gpu_device):
-    """R = 40960 > one-workgroup limit: histogram / scan / rank kernels, 8 source ranks."""
+    """R = 40960: histogram launch + rank launch, 8 source ranks."""
     wl = C.generate_workload("prefill_graph", tokens_scale=10240 / 16384)
     cfg = wl.cfg
     # spread the tokens over 8 uneven source ranks
@@ -151,11 +151,27 @@ def test_token_tile_kernel_on_every_size(gpu_device, monkeypatch, name, scale, p
     assert_same("y", y, o["y"])
 
 
-def test_huge_routing_table(gpu_device):
-    """R = 264000 routed rows: more tiles than the rank kernel sums by itself, so the
-    column-scan kernel runs too."""
+@pytest.mark.parametrize("T,K", [(1001, 3), (2731, 6), (10921, 3), (16383, 3)])
+def test_routing_table_not_a_multiple_of_four(gpu_device, T, K):
+    """The one-launch routing reads the table four entries at a time: R % 4 = 3, 2, 3 (the largest
+    table it takes) and 1 (two launches), separate routing and the fused forms."""
+    g = torch.Generator().manual_seed(T)
+    E, H = 64, 64
+    cfg = C.MoEConfig(E, K, H, T + 1, torch.bfloat16, torch.bfloat16)
+    idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    cuts = [0, T // 3, T // 3, T - 5, T]
+    world = [C.RankData(cuts[i + 1] - cuts[i], idx[cuts[i]:cuts[i + 1]], torch.rand(cuts[i + 1] - cuts[i], K, generator=g),
+                        torch.randn(cuts[i + 1] - cuts[i], H, generator=g).to(torch.bfloat16)) for i in range(4)]
+    for fuse in (False, True):
+        compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=fuse)
+
+
+@pytest.mark.parametrize("T", [12000, 33000])
+def test_huge_routing_table(gpu_device, T):
+    """R = 96000 routed rows: histogram launch + rank launch that scans the tile counts itself;
+    R = 264000: more tiles than the rank kernel sums by itself, so the column-scan kernel runs too."""
     g = torch.Generator().manual_seed(9)
-    T, K, E, H = 33000, 8, 32, 64
+    K, E, H = 8, 32, 64
     cfg = C.MoEConfig(E, K, H, T + 1, torch.float16, torch.float16)
     idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
     world = [C.RankData(T, idx, torch.rand(T, K, generator=g), torch.randn(T, H, generator=g).to(torch.float16))]
