@@ -74,15 +74,19 @@ def parse_args():
     return p.parse_args()
 
 
-def kernel_times(lib, run_n, steps, torch, before_each=None):
+def kernel_times(lib, run_n, steps, torch, before_each=None, lead=0):
     """Per-kernel GPU durations (µs) of `steps` passes launched back to back from C, from the
-    library's launch timer (HIP events bound to each launch)."""
-    cap = steps * 8
+    library's launch timer (HIP events bound to each launch).  `lead` more passes go first in the
+    same loop and are dropped: issuing a timed launch takes the host less time than the GPU needs
+    to run it, so after them the host is a few milliseconds ahead and a host thread that is
+    descheduled for a moment no longer lets the queue run dry in the middle of the timed passes
+    (a kernel that starts on an idle GPU measures 9-18 µs instead of 7)."""
+    cap = (steps + lead) * 8
     rc = lib.moe_a2a_timer_begin(cap)
     if rc != 0:
         raise RuntimeError(f"moe_a2a_timer_begin: {lib.moe_a2a_strerror(rc).decode()}")
     if before_each is None:
-        run_n(steps)
+        run_n(lead + steps)
     else:
         for _ in range(steps):
             before_each()
@@ -94,6 +98,8 @@ def kernel_times(lib, run_n, steps, torch, before_each=None):
     per = {}
     for i in range(n):
         per.setdefault(lib.moe_a2a_kernel_name(ids[i]).decode(), []).append(float(us[i]))
+    if lead:  # every pass launches the same kernels: keep the last `steps` passes of each
+        per = {k: v[len(v) * lead // (lead + steps):] for k, v in per.items()}
     return per
 
 
@@ -214,8 +220,10 @@ def main():
         main.synchronize()
         # the first pass only populates the runtime's pool of events and completion signals
         # (creating them costs driver calls that land in the middle of the launch sequence)
-        kernel_times(lib, run_n, args.steps, torch)
-        per = kernel_times(lib, run_n, args.steps, torch)
+        # untimed passes in front of the timed ones: the W warm-up steps, or about 4 ms of them
+        lead = max(args.warmup, min(300, int(4.0 / ms_per_step)))
+        kernel_times(lib, run_n, args.steps, torch, lead=lead)
+        per = kernel_times(lib, run_n, args.steps, torch, lead=lead)
         if args.dump_times:
             with open(args.dump_times, "w") as f:
                 json.dump(per, f)
@@ -279,7 +287,7 @@ def main():
             run32 = c_loop(step32)
             run32(4)
             main.synchronize()
-            per32 = kernel_times(lib, run32, args.steps, torch)
+            per32 = kernel_times(lib, run32, args.steps, torch, lead=lead)
         t32 = (per_step(per32, ROUTE_KERNELS, args.steps) + per_step(per32, DISPATCH_KERNELS, args.steps) +
                per_step(per32, COMBINE_KERNELS, args.steps))
         out["f32_combine"] = dict(dispatch_combine_us=round(t32, 3),
