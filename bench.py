@@ -35,12 +35,17 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch), each scaled by what the same counter reads for a plain 256 MiB device copy
 # (FETCH_SIZE reads 0.5x the copied bytes there, WRITE_SIZE 1.0x).  Recorded measurements: the
-# commands and raw readings are in profiles/pmc_traffic_dsv3_rank_prefill_graph.txt.
+# commands and raw readings are in profiles/pmc_traffic_dsv3_rank_prefill_graph.txt and
+# profiles/pmc_traffic_skew_world_fp8_dispatch.txt.
 MEASURED_TRAFFIC_BYTES = {
     ("dsv3_rank", "route_dispatch"): int((2.0 * 1850.8 + 28813.3) * 1024),
     ("dsv3_rank", "combine_rows"): int((2.0 * 14426.5 + 3584.0) * 1024),
     ("prefill_graph", "dispatch_rows"): int((2.0 * 66571.0 + 524288.0) * 1024),
     ("prefill_graph", "combine_rows"): int((2.0 * 264208.5 + 131072.0) * 1024),
+    ("skew_world", "route_dispatch_tile"): int((2.0 * 2193.25 + 24937.9) * 1024),
+    ("skew_world", "combine_rows"): int((2.0 * 12458.0 + 4096.0) * 1024),
+    ("fp8_dispatch", "dispatch_fp8"): int((2.0 * 28981.75 + 236544.0) * 1024),
+    ("fp8_dispatch", "combine_rows"): int((2.0 * 230430.5 + 57344.0) * 1024),
 }
 METRIC = "dispatch+combine µs and achieved HBM GB/s (% of peak), 256E/top8/h7168 bf16"
 
