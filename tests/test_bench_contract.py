@@ -1,0 +1,55 @@
+"""bench.py's command line and its one JSON line: the keys a driver reads, the two extra objects,
+and the refusal of more than one GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BENCH = os.path.join(ROOT, "bench.py")
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    p = subprocess.run([sys.executable, BENCH, "--gpus", "2"], capture_output=True, text=True, cwd=ROOT)
+    assert p.returncode != 0
+    assert "one GPU" in p.stderr and "--gpus 2" in p.stderr
+    assert p.stdout.strip() == ""  # no JSON line that a driver could take for a measurement
+
+
+def test_without_a_gpu_the_bench_fails_instead_of_measuring_the_cpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("needs a machine without a GPU")
+    p = subprocess.run([sys.executable, BENCH, "--steps", "2", "--warmup", "1"], capture_output=True, text=True,
+                       cwd=ROOT)
+    assert p.returncode != 0
+    assert p.stdout.strip() == ""
+
+
+@pytest.mark.gpu
+def test_json_line_has_the_contract_keys(gpu_device):
+    p = subprocess.run([sys.executable, BENCH, "--steps", "20", "--warmup", "4", "--cpu-seconds", "1"],
+                       capture_output=True, text=True, cwd=ROOT, timeout=110)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [ln for ln in p.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1, lines
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 20 and d["warmup"] == 4
+    assert d["unit"] == "GB/s" and d["higher_is_better"] is True and d["vs_baseline"] is None
+    assert d["data"] == "synthetic" and d["dtype"] == "bf16"
+    assert d["config"]["workload"] == "dsv3_rank" and "model" not in d["config"]
+    r = d["roofline"]
+    assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
+    assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
+    assert r["traffic"] is None or r["traffic"] > 0
+    # the kernel-time figure cannot beat the memory system, and a step's wall time holds its kernels
+    assert 0 < d["value"] < 8000.0
+    assert d["ms_per_step"] * 1e3 >= d["dispatch_combine_us"]
+    c = d["cpu_baseline"]
+    assert c["kind"] in ("port", "reference") and c["cores"] >= 1 and c["value"] > 0 and c["sample"]
+    assert c["gpu_output_bit_identical"] is True
