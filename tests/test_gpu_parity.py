@@ -198,6 +198,25 @@ def test_fp8_dispatch_power_of_two_scales(gpu_device):
     assert_same("y (forward)", y, o["y"])
 
 
+@pytest.mark.parametrize("H,T,K,E", [(128, 37, 2, 8), (384, 300, 3, 16), (8320, 64, 4, 32), (16384, 33, 8, 64),
+                                     (2048, 1500, 6, 64)])
+@pytest.mark.parametrize("fp8", [True, "pow2"], ids=["f32scales", "pow2scales"])
+def test_fp8_dispatch_row_lengths(gpu_device, H, T, K, E, fp8):
+    """fp8 dispatch on rows of one block, of a few blocks, of more blocks than one workgroup holds
+    (65 and 128: the row is cut in two, each part writes its own scales) and on a table that takes the
+    multi-workgroup routing; ragged world of four ranks."""
+    g = torch.Generator().manual_seed(H + T)
+    cfg = C.MoEConfig(E, K, H, T + 1, torch.bfloat16, torch.bfloat16)
+    idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    x = (torch.randn(T, H, generator=g) * torch.rand(T, 1, generator=g) * 8).to(torch.bfloat16)
+    x[::7, : H // 2] = 0  # whole blocks of zeros: scale 1
+    cuts = [0, T // 4, T // 4, T - 1, T]
+    world = [C.RankData(cuts[i + 1] - cuts[i], idx[cuts[i]:cuts[i + 1]], torch.rand(cuts[i + 1] - cuts[i], K, generator=g),
+                        x[cuts[i]:cuts[i + 1]]) for i in range(4)]
+    compare(cfg, world, gpu_device, C.STUB_EXPERT_FRACTION, fp8=fp8)
+    compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fp8=fp8, combine_mode=C.COMBINE_F32, fuse_route=False)
+
+
 def test_duplicate_experts_and_ragged_world(gpu_device):
     """A token may name the same expert twice; ranks may be empty; H not a multiple of 256 lanes."""
     g = torch.Generator().manual_seed(5)
