@@ -40,6 +40,10 @@ def custom_kernel(data, stub_kind: int = STUB_OWNER_RANK, combine_mode: int = CO
     # the caller owns its result (eval.py deletes it after each run): the combine writes straight
     # into a fresh tensor instead of one of the reused buffers
     y = torch.empty(T, cfg.hidden_dim, dtype=cfg.out_dtype, device=x.device)
-    with torch.cuda.device(x.device):
-        ata.forward(x.contiguous(), rank_data.indices.contiguous(), rank_data.weights.contiguous(), out=y)
+    args = (x.contiguous(), rank_data.indices.contiguous(), rank_data.weights.contiguous())
+    if x.device.index == torch.cuda.current_device():  # the usual case: no device switch to pay for
+        ata.forward(*args, out=y)
+    else:
+        with torch.cuda.device(x.device):
+            ata.forward(*args, out=y)
     return y[: rank_data.num_tokens]
