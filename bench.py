@@ -136,8 +136,10 @@ def c_loop(step):
 
 
 def summarise(per):
-    return {k: dict(mean_us=round(statistics.fmean(v), 3), min_us=round(min(v), 3),
-                    median_us=round(statistics.median(v), 3), launches=len(v)) for k, v in per.items()}
+    return {k: dict(mean_us=round(statistics.fmean(v), 3), std_us=round(statistics.pstdev(v), 3),
+                    err_us=round(statistics.pstdev(v) / max(1, len(v)) ** 0.5, 4), min_us=round(min(v), 3),
+                    max_us=round(max(v), 3), median_us=round(statistics.median(v), 3), launches=len(v))
+            for k, v in per.items()}
 
 
 ROUTE_KERNELS = ("route_tiles", "route_hist", "route_scan", "route_rank")
