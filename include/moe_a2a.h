@@ -222,12 +222,13 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
  * (dequantised and rounded once to elem_type inside the kernel); y[rows, N] of elem_type.
  * Kd % 128 == 0, N % 128 == 0.  Three kernels, chosen by the mean segment length and the rows:
  *   R <= 32 * E (a decode step, bound by the weight bytes, which cross memory once at one byte per
- *     element): 32 x 128 tiles.  16-bit rows: the weight bytes enter the matrix cores exactly (as
- *     16-bit values), each 128-wide K block is summed in f32 and scaled in f32: y = sum over K
- *     blocks of scale_b * (x . q_b).  fp8 rows: the bytes of both operands go memory -> LDS ->
- *     fp8 matrix instruction untouched (the weights with non-temporal loads: they are read once),
- *     folded per K block as below.  MOE_A2A_F8_STREAM=0 sends fp8 rows through the 16-bit form
- *     (dequantised and rounded once to elem_type first).
+ *     element): 32 x 128 tiles, the operand slabs travel memory -> LDS directly (the weights with
+ *     non-temporal loads: they are read once).  16-bit rows: the weight bytes enter the matrix
+ *     cores exactly (turned into 16-bit values in registers), each 128-wide K block is summed in
+ *     f32 and scaled in f32: y = sum over K blocks of scale_b * (x . q_b).  fp8 rows: the bytes of
+ *     both operands go to the fp8 matrix instruction untouched, folded per K block as below.
+ *     MOE_A2A_Q8_STREAM=0 / MOE_A2A_F8_STREAM=0 select the register-staged form of the same
+ *     arithmetic (fp8 rows are then dequantised and rounded once to elem_type first).
  *   longer segments, fp8 rows: both operands enter the fp8 matrix instruction as bytes
  *     (v_mfma_f32_32x32x64_f8f6f4), each 128-wide K block is summed in f32 and folded with
  *     x_scale[row][kb] * w_scale[n / 128][kb]; nothing is rounded before the output.

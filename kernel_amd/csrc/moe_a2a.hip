@@ -818,6 +818,18 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
     return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_f8s_kernel<F16>, grid, block, 0, stream, (const uint4*)x, x_scale,
                   (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
   }
+  if (!x_scale && !(getenv("MOE_A2A_Q8_STREAM") && atoi(getenv("MOE_A2A_Q8_STREAM")) == 0)) {
+    // 16-bit rows: the slabs stream memory -> LDS, the weight bytes become 16-bit fragments in registers
+    const int ntile_n = N / kF8sN;
+    const long long mtiles = (long long)R / kF8sM + E;
+    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
+    dim3 grid((unsigned)(mtiles * ntile_n)), block(kF8sThreads);
+    if (elem_type == MOE_A2A_BF16)
+      return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_q8s_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
+                    (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+    return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_q8s_kernel<F16>, grid, block, 0, stream, (const uint4*)x,
+                  (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
+  }
   const int ntile_n = N / 128;
   const long long mtiles = (long long)R / kSkinnyM + E;
   if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
