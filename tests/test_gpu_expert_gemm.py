@@ -170,15 +170,19 @@ def test_decode_shape_takes_the_skinny_kernel(gpu_device, monkeypatch):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("fp8_rows", [False, True], ids=["rows16", "rows8"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-@pytest.mark.parametrize("tile", ["32", "128", "256"], ids=["tile32", "tile128", "tile256"])
+@pytest.mark.parametrize("tile", ["32", "32r", "128", "256"], ids=["tile32", "tile32staged", "tile128", "tile256"])
 def test_expert_gemm_block_quantised_weights(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, fp8_rows,
                                              padded, tile):
     """Weights as e4m3fn bytes with one scale per 128 x 128 block, rows 16-bit or from the fp8
     dispatch, against an f32 matmul of the dequantised operands (each rounded once to the 16-bit
     type, as two of the kernels do), through the weight-streaming kernel, the fp8 x fp8 kernel (tile
     128, fp8 rows only: 16-bit rows keep the default choice) and the 256 x 256 kernel (which needs
-    N >= 256; the one N == 128 case stays on the other)."""
-    monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile)
+    N >= 256; the one N == 128 case stays on the other).  The weight-streaming form exists twice:
+    slabs sent memory -> LDS directly (tile32) and staged through registers (tile32staged)."""
+    monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile[:2] if tile.startswith("32") else tile)
+    if tile == "32r":
+        monkeypatch.setenv("MOE_A2A_Q8_STREAM", "0")
+        monkeypatch.setenv("MOE_A2A_F8_STREAM", "0")
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=5 * E + T, zipf=zipf)
     wq, ws = V.quantize_weights_fp8(weights)
     x, idx, w, rs = concat_world(world, gpu_device)
