@@ -79,19 +79,30 @@ def parse_args():
     return p.parse_args()
 
 
-def kernel_times(lib, run_n, steps, torch, before_each=None, lead=0):
+def kernel_times(lib, run_n, steps, torch, before_each=None, lead=0, launches_per_step=0, wall=None):
     """Per-kernel GPU durations (µs) of `steps` passes launched back to back from C, from the
-    library's launch timer (HIP events bound to each launch).  `lead` more passes go first in the
-    same loop and are dropped: issuing a timed launch takes the host less time than the GPU needs
-    to run it, so after them the host is a few milliseconds ahead and a host thread that is
-    descheduled for a moment no longer lets the queue run dry in the middle of the timed passes
-    (a kernel that starts on an idle GPU measures 9-18 µs instead of 7)."""
-    cap = (steps + lead) * 8
+    library's launch timer (HIP events bound to each launch).  `lead` passes go first in the same
+    loop WITHOUT events: a launch that carries events costs the host about 13 µs, a plain one
+    2.5 µs, a small kernel runs 7 µs -- the plain passes put the host ahead, so that the timed ones
+    find the queue full and run back to back as in a hipGraph replay.  `wall = (stream, list)`
+    appends the wall clock per step of the timed passes themselves (an upper bound for the sum of
+    their kernels)."""
+    cap = steps * 8
     rc = lib.moe_a2a_timer_begin(cap)
     if rc != 0:
         raise RuntimeError(f"moe_a2a_timer_begin: {lib.moe_a2a_strerror(rc).decode()}")
     if before_each is None:
-        run_n(lead + steps)
+        if lead:
+            lib.moe_a2a_timer_skip(lead * launches_per_step)
+            run_n(lead)
+        if wall is not None:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(wall[0])
+        run_n(steps)
+        if wall is not None:
+            e1.record(wall[0])
+            torch.cuda.synchronize()
+            wall[1].append(e0.elapsed_time(e1) * 1e3 / steps)
     else:
         for _ in range(steps):
             before_each()
@@ -103,9 +114,28 @@ def kernel_times(lib, run_n, steps, torch, before_each=None, lead=0):
     per = {}
     for i in range(n):
         per.setdefault(lib.moe_a2a_kernel_name(ids[i]).decode(), []).append(float(us[i]))
-    if lead:  # every pass launches the same kernels: keep the last `steps` passes of each
-        per = {k: v[len(v) * lead // (lead + steps):] for k, v in per.items()}
     return per
+
+
+def lead_passes(lib, run_n, steps, gpu_step_us, torch, floor):
+    """How many plain passes must go first so that the queue outlasts `steps` timed passes: measures
+    what a plain and a timed pass cost the host (µs) and how many launches a pass holds."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_n(20)
+    plain = (time.perf_counter() - t0) / 20 * 1e6
+    torch.cuda.synchronize()
+    lib.moe_a2a_timer_begin(20 * 8)
+    t0 = time.perf_counter()
+    run_n(20)
+    timed = (time.perf_counter() - t0) / 20 * 1e6
+    torch.cuda.synchronize()
+    ids, us = (ctypes.c_int * 160)(), (ctypes.c_float * 160)()
+    launches = lib.moe_a2a_timer_end(ids, us, 160) // 20
+    deficit = max(0.0, timed - gpu_step_us) * steps
+    gain = max(gpu_step_us - plain, 0.1 * gpu_step_us)
+    lead = int(1.3 * deficit / gain) + 1
+    return max(floor, min(lead, 2000)), launches, plain, timed
 
 
 class ForwardArgs(ctypes.Structure):
@@ -227,13 +257,16 @@ def main():
         main.synchronize()
         # the first pass only populates the runtime's pool of events and completion signals
         # (creating them costs driver calls that land in the middle of the launch sequence)
-        # untimed passes in front of the timed ones: the W warm-up steps, or about 4 ms of them
-        lead = max(args.warmup, min(300, int(4.0 / ms_per_step)))
-        kernel_times(lib, run_n, args.steps, torch, lead=lead)
-        per = kernel_times(lib, run_n, args.steps, torch, lead=lead)
+        # plain passes in front of the timed ones: at least the W warm-up steps
+        lead, n_launch, host_plain_us, host_timed_us = lead_passes(lib, run_n, args.steps, ms_per_step * 1e3, torch,
+                                                                   args.warmup)
+        kernel_times(lib, run_n, args.steps, torch, lead=lead, launches_per_step=n_launch)
+        pass_wall = []
+        per = kernel_times(lib, run_n, args.steps, torch, lead=lead, launches_per_step=n_launch,
+                           wall=(main, pass_wall))
         if args.dump_times:
             with open(args.dump_times, "w") as f:
-                json.dump(per, f)
+                json.dump({**per, "_wall_us_per_step_of_the_timed_passes": pass_wall}, f)
         e0.record(main)
         run_n(timed_steps)
         e1.record(main)
@@ -275,6 +308,8 @@ def main():
         tokens_per_s=round(T / (t_dc * 1e-6), 1),
         tokens_per_s_wall=round(T / (ms_per_step * 1e-3), 1),
         eager_ms_per_step=round(eager_ms_per_step, 6),
+        timed_passes=dict(wall_us_per_step=round(pass_wall[0], 3), plain_lead_passes=lead,
+                          host_us_per_plain_pass=round(host_plain_us, 2), host_us_per_timed_pass=round(host_timed_us, 2)),
         bytes=dict(dispatch=ab["dispatch"], combine=ab["combine"], stub=ab["stub"]),
         kernels=summarise(per),
         roofline=roofline,
@@ -294,7 +329,7 @@ def main():
             run32 = c_loop(step32)
             run32(4)
             main.synchronize()
-            per32 = kernel_times(lib, run32, args.steps, torch, lead=lead)
+            per32 = kernel_times(lib, run32, args.steps, torch, lead=lead, launches_per_step=n_launch)
         t32 = (per_step(per32, ROUTE_KERNELS, args.steps) + per_step(per32, DISPATCH_KERNELS, args.steps) +
                per_step(per32, COMBINE_KERNELS, args.steps))
         out["f32_combine"] = dict(dispatch_combine_us=round(t32, 3),

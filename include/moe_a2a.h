@@ -269,9 +269,13 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
  *   begin(capacity)  allocate `capacity` event pairs and start recording
  *   end(ids, us, n)  wait for the recorded launches, write up to n (kernel id, microseconds)
  *                    pairs to HOST arrays, release the events; returns the number written
+ *   skip(launches)   the next `launches` launches go out without events (they cost the host a
+ *                    fifth of a timed launch: a caller issues untimed steps first so that the GPU
+ *                    queue stays full while the timed ones are issued)
  *   kernel_name(id)  host string for a kernel id
  */
 int moe_a2a_timer_begin(int capacity);
+int moe_a2a_timer_skip(int launches);
 int moe_a2a_timer_end(int* kernel_ids, float* microseconds, int n);
 const char* moe_a2a_kernel_name(int kernel_id);
 

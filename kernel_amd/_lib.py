@@ -41,6 +41,7 @@ PROTOTYPES = {
     "moe_a2a_expert_gemm_q8": (_int, [_vp, _vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_expert_gemm_mx8": (_int, [_vp, _vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_timer_begin": (_int, [_int]),
+    "moe_a2a_timer_skip": (_int, [_int]),
     "moe_a2a_timer_end": (_int, [C.POINTER(C.c_int), C.POINTER(C.c_float), _int]),
     "moe_a2a_kernel_name": (C.c_char_p, [_int]),
 }
