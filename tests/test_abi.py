@@ -158,6 +158,7 @@ def test_timer_needs_begin_first(lib):
     ids = (ctypes.c_int * 4)()
     us = (ctypes.c_float * 4)()
     assert lib.moe_a2a_timer_end(ids, us, 4) == E_STATE
+    assert lib.moe_a2a_timer_skip(3) == E_STATE
     assert lib.moe_a2a_timer_begin(0) == E_STATE
 
 

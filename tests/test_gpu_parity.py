@@ -151,6 +151,29 @@ def test_token_tile_kernel_on_every_size(gpu_device, monkeypatch, name, scale, p
     assert_same("y", y, o["y"])
 
 
+def test_launch_timer_skips_the_launches_it_is_told_to(gpu_device):
+    """Launches skipped by moe_a2a_timer_skip go out without events: they are not reported, the
+    ones after them are, and every result is what it would be without the timer."""
+    import ctypes
+    wl = C.generate_workload("dsv3_rank", tokens_scale=0.25)
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    ata = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind)
+    lib = ata.lib
+    o = V.run_world(wl.cfg, wl.world, stub_kind=wl.stub_kind)
+    assert lib.moe_a2a_timer_begin(16) == 0
+    assert lib.moe_a2a_timer_skip(-1) != 0
+    assert lib.moe_a2a_timer_skip(3) == 0  # one forward: route_dispatch, stub, combine
+    y1 = ata.forward(x, idx, w, rs).clone()
+    y2 = ata.forward(x, idx, w, rs).clone()
+    torch.cuda.synchronize()
+    ids, us = (ctypes.c_int * 16)(), (ctypes.c_float * 16)()
+    assert lib.moe_a2a_timer_end(ids, us, 16) == 3
+    assert [lib.moe_a2a_kernel_name(ids[i]) for i in range(3)] == [b"route_dispatch", b"stub_rows", b"combine_rows"]
+    assert all(0.5 < us[i] < 1000 for i in range(3))
+    assert_same("y (skipped)", y1, o["y"])
+    assert_same("y (timed)", y2, o["y"])
+
+
 @pytest.mark.parametrize("T,K", [(1001, 3), (2731, 6), (10921, 3), (16383, 3)])
 def test_routing_table_not_a_multiple_of_four(gpu_device, T, K):
     """The one-launch routing reads the table four entries at a time: R % 4 = 3, 2, 3 (the largest
