@@ -229,9 +229,16 @@ def main():
                 step()
                 y = step()
             run = graph.replay
+            graph1 = None
+            if args.steps % 2:  # an odd K ends with one single-step graph, so that exactly K steps are timed
+                graph1 = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph1, stream=main):
+                    y = step()
 
-        n_runs = max(1, args.steps // steps_per_run)
-        timed_steps = n_runs * steps_per_run
+        if args.steps < 1:
+            raise SystemExit("--steps must be at least 1")
+        n_runs = args.steps // steps_per_run
+        timed_steps = args.steps
         # spin-up: the first milliseconds of GPU work after an idle period run below the
         # sustained clocks; 0.3 s of untimed steps come before the W warm-up steps
         t_spin = time.perf_counter()
@@ -246,6 +253,8 @@ def main():
         e0.record(main)
         for _ in range(n_runs):
             run()
+        if use_graph and graph1 is not None:
+            graph1.replay()
         e1.record(main)
         main.synchronize()
         ms_per_step = e0.elapsed_time(e1) / timed_steps
