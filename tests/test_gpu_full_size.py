@@ -108,6 +108,48 @@ def test_round_trip_and_checksums(gpu_device, name):
         assert torch.equal(bits(getattr(d2, k)), bits(v)), k
 
 
+def test_buffers_beyond_four_gigabytes(gpu_device):
+    """304 000 routed rows of 7168 columns: 2.2e9 elements, 4.4 GB per row buffer, so element and
+    byte offsets leave the 32-bit range (and the table takes the three-launch routing).  No oracle:
+    round trip with one-hot weights, routing invariants, checksum of checksums, fp8 bound on the
+    last rows."""
+    T, K, E, H = 38000, 8, 64, 7168
+    cfg = C.MoEConfig(E, K, H, T + 1, torch.bfloat16, torch.bfloat16)
+    g = torch.Generator(device=gpu_device).manual_seed(5)
+    x = torch.randn(T, H, generator=g, device=gpu_device).to(torch.bfloat16)
+    idx = torch.rand(T, E, generator=g, device=gpu_device).topk(K, dim=1).indices.to(torch.int32)  # distinct per token
+    hot = torch.randint(0, K, (T,), generator=g, device=gpu_device)
+    w1 = torch.nn.functional.one_hot(hot, K).float()
+    ata = HipAllToAll(cfg, 0, 1, stub_kind=C.STUB_OWNER_RANK)  # one emulated rank: the stub factor is 1
+    R = T * K
+    assert R * H > 2 ** 31
+    for mode in (C.COMBINE_STRICT, C.COMBINE_F32):
+        ata.combine_mode = mode
+        y = ata.forward(x, idx, w1)
+        assert torch.equal(y.view(torch.int16), x.view(torch.int16))
+    d = ata.last
+    assert int(d.status.item()) == 0
+    assert int(d.counts.sum()) == R and int(d.offsets[-1]) == R
+    assert torch.equal(d.src_of_slot[d.slot_of_entry.long()], torch.arange(R, dtype=torch.int32, device=gpu_device))
+    assert torch.equal(d.meta[:, 0], idx.flatten()[d.src_of_slot.long()])
+    row_sum = x.view(torch.int16).sum(dim=1, dtype=torch.int64)
+    disp_sum = d.disp_x.view(torch.int16).sum(dim=1, dtype=torch.int64)
+    assert torch.equal(disp_sum, row_sum[d.src_of_slot.long() // K])
+    ata.release_buffers()
+    del y, d
+    # fp8 dispatch of the same rows: the last 4096 rows of the buffer (beyond 2^31 bytes) obey the bound
+    ata8 = HipAllToAll(cfg, 0, 1, stub_kind=C.STUB_OWNER_RANK, fp8_dispatch=True)
+    d8 = ata8.dispatch(x, idx)
+    torch.cuda.synchronize()
+    rows = torch.arange(R - 4096, R, device=gpu_device)
+    q = d8.disp_x[rows].view(torch.float8_e4m3fn).float().view(4096, H // 128, 128)
+    sc = d8.disp_scale[rows].view(4096, H // 128, 1)
+    xs = x[d8.src_of_slot[rows].long() // K].float().view(4096, H // 128, 128)
+    bound = torch.maximum(xs.abs() * 2.0 ** -4, sc * 2.0 ** -10) * (1 + 1e-6)
+    assert bool(((q * sc - xs).abs() <= bound).all())
+    ata8.release_buffers()
+
+
 def test_linearity_of_combine_in_the_weights(gpu_device):
     """f32-mode combine is linear in the weights up to rounding: y(w) + y(w') ~ y(w + w')."""
     wl = C.generate_workload("skew_world")
