@@ -156,7 +156,9 @@ int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta,
  * (all2all/reference.py:163-232 without the regroup/exchange).  STRICT reproduces the
  * reference's order (ascending slot) and its rounding to the output type after every add;
  * F32 keeps an f32 accumulator in k order.  Multiply and add are never contracted.
- * Rows of out that belong to no token are not touched.
+ * Rows of out that belong to no token are not touched.  (Cache policy of the output stores at
+ * streaming sizes: this entry point does not know what the dispatch wrote and assumes one byte
+ * per element of the expert rows; moe_a2a_forward decides from the actual figure.)
  */
 int moe_a2a_combine(const void* expert_y, const float* weights, const int32_t* slot_of_entry, int mode,
                     int elem_type, void* out, int T, int K, int H, moe_a2a_stream_t stream);

@@ -47,6 +47,18 @@ def test_full_size_against_oracle(gpu_device, name):
     # the stub folded into the combine gives the same bits
     _, _, y2, _ = gpu_run(wl, gpu_device, fuse_stub=True)
     assert torch.equal(bits(y2.cpu()), bits(want["y"]))
+    # the one-call forward knows what the dispatch wrote and may pick other cache policies for the
+    # combine (write-through output stores beyond 256 MB of dispatched rows): same bits, both modes
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    for mode in (C.COMBINE_STRICT, C.COMBINE_F32):
+        ata.combine_mode = mode
+        y3 = ata.forward(x, idx, w, rs)
+        torch.cuda.synchronize()
+        if mode == C.COMBINE_STRICT:
+            assert torch.equal(bits(y3.cpu()), bits(want["y"]))
+        else:
+            want32 = V.run_world(wl.cfg, wl.world, stub_kind=wl.stub_kind, fp8=wl.fp8_dispatch, combine_mode=mode)["y"]
+            assert torch.equal(bits(y3.cpu()), bits(want32))
 
 
 def test_fp8_rows_within_stated_bound_at_full_size(gpu_device):
