@@ -3,18 +3,22 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload dsv3_rank]
 
-A step is one pass of the path over one resident batch: routing + dispatch, expert stub,
-combine (three launches at the default workload), replayed from a hipGraph.  Inputs are in
-HBM before the timed region starts.  Prints ONE JSON line:
+A step is one pass of the path over one resident batch, in the configuration `custom_kernel`
+runs: routing + dispatch in one launch, then the combine with the expert stand-in folded in (two
+launches at the default workload), replayed from a hipGraph.  Inputs are in HBM before the timed
+region starts.  Prints ONE JSON line:
 
   value        achieved GB/s of dispatch+combine: algorithmic bytes (read x once, write R
                rows; read R rows, write T rows) / summed GPU durations of the routing,
                dispatch and combine kernels of a step.  Kernel durations come from HIP
                events bound to each launch, on the stream the kernels run on.
-  ms_per_step  wall time of a whole step (including the stub launch), events around K steps.
-  roofline     the slower of the dispatch / combine kernels against the 8 TB/s HBM peak.
+  ms_per_step  wall time of a whole step, events around K steps of hipGraph replays.
+  roofline     the slower of the dispatch / combine kernels against the 8 TB/s HBM peak; `traffic`
+               from profiles/traffic.json when that record was taken on the present kernel sources.
   cpu_baseline the CPU oracle (a port of the reference's torch path) timed on the host
                cores for the same workload, and used to check the GPU result.
+Beside the headline: the same path with the stub as a launch of its own, and with the
+f32-accumulating combine.  `--graph-only` runs the graph replays and nothing else (for rocprofv3).
 """
 from __future__ import annotations
 
@@ -32,21 +36,46 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch), each scaled by what the same counter reads for a plain 256 MiB device copy
-# (FETCH_SIZE reads 0.5x the copied bytes there, WRITE_SIZE 1.0x).  Recorded measurements: the
-# commands and raw readings are in profiles/pmc_traffic_dsv3_rank_prefill_graph.txt and
-# profiles/pmc_traffic_skew_world_fp8_dispatch.txt.
-MEASURED_TRAFFIC_BYTES = {
-    ("dsv3_rank", "route_dispatch"): int((2.0 * 1850.8 + 28813.3) * 1024),
-    ("dsv3_rank", "combine_rows"): int((2.0 * 14426.5 + 3584.0) * 1024),
-    ("prefill_graph", "dispatch_rows"): int((2.0 * 66571.0 + 524288.0) * 1024),
-    ("prefill_graph", "combine_rows"): int((2.0 * 264208.5 + 131072.0) * 1024),
-    ("skew_world", "route_dispatch_tile"): int((2.0 * 2193.25 + 24937.9) * 1024),
-    ("skew_world", "combine_rows"): int((2.0 * 12458.0 + 4096.0) * 1024),
-    ("fp8_dispatch", "dispatch_fp8"): int((2.0 * 28981.75 + 236544.0) * 1024),
-    ("fp8_dispatch", "combine_rows"): int((2.0 * 230430.5 + 57344.0) * 1024),
-}
+# HBM bytes per launch, measured: profiles/traffic.json holds rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# readings (KiB per dispatch, each scaled by what the same counter reads for a plain 256 MiB device
+# copy) together with the kernel's name and a hash of the kernel sources they were taken from.
+# `python bench.py --record-traffic DIR` writes that file from the CSVs of such runs.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_SOURCES = ("kernel_amd/csrc/moe_a2a.hip", "kernel_amd/csrc/route_kernels.inc", "kernel_amd/csrc/row_kernels.inc")
+
+
+def kernel_source_hash():
+    """sha256 over the sources of the dispatch / combine kernels: a traffic record counts only for
+    the code it was measured on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, kernel, path=TRAFFIC_FILE, source_hash=None):
+    """(bytes per launch or None, where the figure comes from / why there is none)."""
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, "no traffic record (profiles/traffic.json missing or unreadable)"
+    source_hash = source_hash or kernel_source_hash()
+    for e in rec.get("entries", []):
+        if e.get("workload") == workload and e.get("kernel") == kernel:
+            if e.get("source_hash") != source_hash:
+                return None, (f"record of {kernel} at {workload} was measured on other kernel sources "
+                              f"({e.get('source_hash')}, now {source_hash}): not reported")
+            return int(e["bytes"]), (f"profiles/traffic.json: rocprofv3 --pmc, {e['fetch_kib']} KiB FETCH_SIZE x "
+                                     f"{rec['factor']['FETCH_SIZE']} + {e['write_kib']} KiB WRITE_SIZE x "
+                                     f"{rec['factor']['WRITE_SIZE']}, kernel {e.get('symbol', kernel)}, "
+                                     f"sources {e['source_hash']}, commit {e.get('commit', '?')}")
+    return None, f"no record of {kernel} at {workload}"
+
+
 METRIC = "dispatch+combine µs and achieved HBM GB/s (% of peak), 256E/top8/h7168 bf16"
 
 
@@ -59,7 +88,17 @@ def parse_args():
     p.add_argument("--combine", choices=["strict", "f32"], default="strict")
     p.add_argument("--no-graph", action="store_true", help="launch eagerly from Python instead of a hipGraph")
     p.add_argument("--no-fuse-route", action="store_true", help="separate routing kernel even for small worlds")
-    p.add_argument("--fuse-stub", action="store_true", help="fold the expert stub into the combine")
+    p.add_argument("--no-fuse-stub", action="store_true",
+                   help="expert stub as a launch of its own (the default folds it into the combine, as custom_kernel does)")
+    p.add_argument("--graph-only", action="store_true",
+                   help="hipGraph replays of the default configuration and nothing else (the form to run under rocprofv3)")
+    p.add_argument("--single", action="store_true", help="skip the legs reported beside the headline (other stub form, f32 combine)")
+    p.add_argument("--timer-event-flags", default="", metavar="FLAGS",
+                   help="hipEventCreateWithFlags value for the launch timer's events (measurement aid)")
+    p.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                   help="library option switch (moe_a2a_set_option), e.g. COMBINE_LANES=128 (measurement aid)")
+    p.add_argument("--record-traffic", metavar="DIR",
+                   help="no measurement: fold rocprofv3 --pmc CSVs under DIR into profiles/traffic.json")
     p.add_argument("--bf16-dispatch", action="store_true", help="fp8 workload with a 16-bit dispatch")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--cold", action="store_true", help="add a leg with caches flushed before every step")
@@ -182,113 +221,179 @@ def per_step(per, names, steps):
     return sum(sum(per.get(n, [])) for n in names) / steps
 
 
+class Leg:
+    """One configuration of the path (host object, planned step, hipGraphs) and its measurements."""
+
+    def __init__(self, torch, lib, wl, tensors, main, mode, fp8, fuse_route, fuse_stub):
+        from kernel_amd.all2all import HipAllToAll
+
+        self.torch, self.lib, self.main = torch, lib, main
+        x, idx, w, rs = tensors
+        self.ata = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind, combine_mode=mode, fp8_dispatch=fp8,
+                               fuse_route=fuse_route, fuse_stub=fuse_stub)
+        with torch.cuda.stream(main):
+            self.step = self.ata.plan(x, idx, w, rs, stream=main)  # pre-marshalled: one foreign call per step
+            self.step()
+            self.y = self.step()  # both buffer sets exist now
+            main.synchronize()
+        self.run_n = None
+
+    def graph_wall(self, steps, warmup, use_graph=True):
+        """Wall time per step (ms) of exactly `steps` steps: hipGraph replays (the host class alternates
+        between two buffer sets, so one graph holds two steps; an odd count ends with a one-step graph)."""
+        torch, main, step = self.torch, self.main, self.step
+        with torch.cuda.stream(main):
+            run, per_run, tail = step, 1, None
+            if use_graph:
+                per_run = 2
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=main):
+                    step()
+                    self.y = step()
+                run = graph.replay
+                if steps % 2:
+                    tail = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(tail, stream=main):
+                        self.y = step()
+            # spin-up: the first milliseconds of GPU work after an idle period run below the
+            # sustained clocks; 0.3 s of untimed steps come before the W warm-up steps
+            t_spin = time.perf_counter()
+            while time.perf_counter() - t_spin < 0.3:
+                for _ in range(50):
+                    run()
+                main.synchronize()
+            for _ in range(max(1, warmup // per_run)):
+                run()
+            main.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(main)
+            for _ in range(steps // per_run):
+                run()
+            if tail is not None:
+                tail.replay()
+            e1.record(main)
+            main.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    def kernels(self, steps, warmup, gpu_step_us, want_wall=False):
+        """Per-kernel durations (us) of `steps` steps launched back to back from C, every launch with
+        its own pair of HIP events; returns (per-kernel lists, details)."""
+        torch, lib, main = self.torch, self.lib, self.main
+        with torch.cuda.stream(main):
+            if self.run_n is None:
+                self.run_n = c_loop(self.step)
+                self.run_n(4)
+                main.synchronize()
+            run_n = self.run_n
+            lead, n_launch, host_plain_us, host_timed_us = lead_passes(lib, run_n, steps, gpu_step_us, torch, warmup)
+            # the first pass only populates the runtime's pool of events and completion signals
+            # (creating them costs driver calls that land in the middle of the launch sequence)
+            kernel_times(lib, run_n, steps, torch, lead=lead, launches_per_step=n_launch)
+            pass_wall = []
+            per = kernel_times(lib, run_n, steps, torch, lead=lead, launches_per_step=n_launch,
+                               wall=(main, pass_wall) if want_wall else None)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(main)
+            run_n(steps)
+            e1.record(main)
+            main.synchronize()
+        details = dict(plain_lead_passes=lead, host_us_per_plain_pass=round(host_plain_us, 2),
+                       host_us_per_timed_pass=round(host_timed_us, 2), launches_per_step=n_launch,
+                       eager_ms_per_step=e0.elapsed_time(e1) / steps)
+        if want_wall:
+            details["wall_us_per_step"] = round(pass_wall[0], 3)
+        return per, details
+
+
+def phase_times(per, steps):
+    t = dict(route=per_step(per, ROUTE_KERNELS, steps), dispatch=per_step(per, DISPATCH_KERNELS, steps),
+             combine=per_step(per, COMBINE_KERNELS, steps), stub=per_step(per, STUB_KERNELS, steps))
+    t["dc"] = t["route"] + t["dispatch"] + t["combine"]
+    return t
+
+
 def main():
     args = parse_args()
+    if args.record_traffic:
+        return record_traffic(args.record_traffic)
     if args.gpus != 1:
         print(f"bench.py measures one GPU: the emulated destination ranks are partitions of one HBM buffer and "
               f"there is no cross-GPU path in this build (got --gpus {args.gpus}).", file=sys.stderr)
         sys.exit(2)
+    if args.steps < 1:
+        raise SystemExit("--steps must be at least 1")
     import torch
 
     from kernel_amd import _lib, contract
-    from kernel_amd.all2all import HipAllToAll, concat_world
+    from kernel_amd.all2all import concat_world
 
     lib = _lib.load()
     if not torch.cuda.is_available():
         raise RuntimeError("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.timer_event_flags:
+        lib.moe_a2a_set_option(_lib.OPT_TIMER_EVENT_FLAGS, int(args.timer_event_flags, 0))
+    for item in args.option:
+        name, _, val = item.partition("=")
+        if lib.moe_a2a_set_option(getattr(_lib, "OPT_" + name), int(val, 0)) < 0:
+            raise SystemExit(f"unknown option {name}")
 
     wl = contract.generate_workload(args.workload)
     cfg, W = wl.cfg, wl.world_size
     T, K, H, E = wl.total_tokens, cfg.experts_per_token, cfg.hidden_dim, cfg.num_experts
     fp8 = wl.fp8_dispatch and not args.bf16_dispatch
     mode = contract.COMBINE_STRICT if args.combine == "strict" else contract.COMBINE_F32
-    ata = HipAllToAll(cfg, 0, W, stub_kind=wl.stub_kind, combine_mode=mode, fp8_dispatch=fp8,
-                      fuse_route=not args.no_fuse_route, fuse_stub=args.fuse_stub)
-    x, idx, w, rs = concat_world(wl.world, dev)
+    fuse_route, fuse_stub = not args.no_fuse_route, not args.no_fuse_stub
+    tensors = concat_world(wl.world, dev)
     if args.expert_gemm:
-        return expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev)
+        return expert_gemm_leg(args, lib, torch, wl, tensors[0], tensors[1], tensors[3], dev)
 
     # Everything runs on one non-blocking stream of its own: launches on the legacy default
     # stream carry implicit waits on every other stream of the process.
     main = torch.cuda.Stream()
     main.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(main):
-        step = ata.plan(x, idx, w, rs, stream=main)  # pre-marshalled: one foreign call per step
-        step()
-        y = step()  # both buffer sets exist now
-        main.synchronize()
-        run, steps_per_run = step, 1
-        use_graph = not args.no_graph
-        if use_graph:
-            # the host class alternates between two buffer sets, so one graph holds two steps
-            steps_per_run = 2
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=main):
-                step()
-                y = step()
-            run = graph.replay
-            graph1 = None
-            if args.steps % 2:  # an odd K ends with one single-step graph, so that exactly K steps are timed
-                graph1 = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph1, stream=main):
-                    y = step()
-
-        if args.steps < 1:
-            raise SystemExit("--steps must be at least 1")
-        n_runs = args.steps // steps_per_run
-        timed_steps = args.steps
-        # spin-up: the first milliseconds of GPU work after an idle period run below the
-        # sustained clocks; 0.3 s of untimed steps come before the W warm-up steps
-        t_spin = time.perf_counter()
-        while time.perf_counter() - t_spin < 0.3:
-            for _ in range(50):
-                run()
-            main.synchronize()
-        for _ in range(max(1, args.warmup // steps_per_run)):
-            run()
-        main.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(main)
-        for _ in range(n_runs):
-            run()
-        if use_graph and graph1 is not None:
-            graph1.replay()
-        e1.record(main)
-        main.synchronize()
-        ms_per_step = e0.elapsed_time(e1) / timed_steps
-
-        # per-kernel durations: the same launches issued back to back from a C loop, each
-        # carrying its own pair of HIP events
-        run_n = c_loop(step)
-        run_n(4)
-        main.synchronize()
-        # the first pass only populates the runtime's pool of events and completion signals
-        # (creating them costs driver calls that land in the middle of the launch sequence)
-        # plain passes in front of the timed ones: at least the W warm-up steps
-        lead, n_launch, host_plain_us, host_timed_us = lead_passes(lib, run_n, args.steps, ms_per_step * 1e3, torch,
-                                                                   args.warmup)
-        kernel_times(lib, run_n, args.steps, torch, lead=lead, launches_per_step=n_launch)
-        pass_wall = []
-        per = kernel_times(lib, run_n, args.steps, torch, lead=lead, launches_per_step=n_launch,
-                           wall=(main, pass_wall))
-        if args.dump_times:
-            with open(args.dump_times, "w") as f:
-                json.dump({**per, "_wall_us_per_step_of_the_timed_passes": pass_wall}, f)
-        e0.record(main)
-        run_n(timed_steps)
-        e1.record(main)
-        main.synchronize()
-        eager_ms_per_step = e0.elapsed_time(e1) / timed_steps
-    t_route = per_step(per, ROUTE_KERNELS, args.steps)
-    t_disp = per_step(per, DISPATCH_KERNELS, args.steps)
-    t_comb = per_step(per, COMBINE_KERNELS, args.steps)
-    t_stub = per_step(per, STUB_KERNELS, args.steps)
     ab = contract.algorithmic_bytes(T, K, H, 2, 2, fp8)
     b_dc = ab["dispatch"] + ab["combine"]
-    t_dc = t_route + t_disp + t_comb
-    value = b_dc / t_dc / 1e3  # bytes/µs -> GB/s
+    use_graph = not args.no_graph
+    dtype = "fp8-e4m3 dispatch, bf16 combine" if fp8 else {"bfloat16": "bf16", "float16": "f16"}[
+        str(cfg.in_dtype).replace("torch.", "")]
+    config = dict(workload=args.workload, tokens=T, experts=E, top_k=K, hidden=H, emulated_ranks=W, routed_rows=T * K,
+                  combine=args.combine,
+                  launch="hipGraph replay, two steps per graph" if use_graph else "eager",
+                  fused_route=bool(fuse_route and not fp8 and lib.moe_a2a_fused_ok(T, K, H)),
+                  fused_stub=bool(fuse_stub),
+                  entry_point="what custom_kernel runs: routing+dispatch, then the combine with the expert stub "
+                              "folded in" if fuse_stub else "routing+dispatch, stub kernel, combine")
+
+    # the configuration custom_kernel runs (kernel_amd/submission.py): the expert stand-in folded
+    # into the combine, two launches per step at the default workload
+    leg = Leg(torch, lib, wl, tensors, main, mode, fp8, fuse_route, fuse_stub)
+    ms_per_step = leg.graph_wall(args.steps, args.warmup, use_graph)
+
+    if args.graph_only:
+        # Nothing but the graph replays above: no event-carrying launch, no second configuration.  This
+        # is the form to put under `rocprofv3 --kernel-trace --stats`, whose per-kernel averages then
+        # describe exactly these launches.  `value` is the wall-clock figure, which includes the idle
+        # time between launches: a lower bound of the kernels' own rate.
+        wall_us = ms_per_step * 1e3
+        out = dict(metric=METRIC, value=round(b_dc / wall_us / 1e3, 1), unit="GB/s", n_gpus=1, steps=args.steps,
+                   warmup=args.warmup, ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak",
+                   vs_baseline=None, dtype=dtype, data="synthetic",
+                   config=dict(config, launch="hipGraph replay only; value from the wall clock of whole steps"),
+                   bytes=dict(dispatch=ab["dispatch"], combine=ab["combine"], stub=ab["stub"]),
+                   roofline=None, cpu_baseline=None)
+        if args.calibrate_copy:
+            calibrate_copy(torch, main, dev)
+        print(json.dumps(out, ensure_ascii=False), flush=True)
+        return
+
+    per, det = leg.kernels(args.steps, args.warmup, ms_per_step * 1e3, want_wall=True)
+    if args.dump_times:
+        with open(args.dump_times, "w") as f:
+            json.dump({**per, "_wall_us_per_step_of_the_timed_passes": [det["wall_us_per_step"]]}, f)
+    t = phase_times(per, args.steps)
+    value = b_dc / t["dc"] / 1e3  # bytes/us -> GB/s
 
     # dominant kernel for the roofline entry
     disp_name = next(n for n in DISPATCH_KERNELS if n in per)
@@ -296,65 +401,60 @@ def main():
     cand = [(disp_name, ab["dispatch"]), (comb_name, ab["combine"])]
     dom_name, dom_bytes = max(cand, key=lambda c: statistics.fmean(per[c[0]]))
     dom_us = statistics.fmean(per[dom_name])
+    traffic, traffic_source = measured_traffic(args.workload, dom_name)
     roofline = dict(bound="hbm", kernel=dom_name, achieved=round(dom_bytes / dom_us / 1e3, 1), peak=HBM_PEAK_GBPS,
                     unit="GB/s", frac=round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
-                    bytes_per_launch=dom_bytes, avg_us=round(dom_us, 3),
-                    traffic=MEASURED_TRAFFIC_BYTES.get((args.workload, dom_name)))
+                    bytes_per_launch=dom_bytes, avg_us=round(dom_us, 3), traffic=traffic,
+                    traffic_source=traffic_source)
 
     out = dict(
-        metric=METRIC, value=round(value, 1), unit="GB/s", n_gpus=1, steps=timed_steps, warmup=args.warmup,
-        ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
-        dtype="fp8-e4m3 dispatch, bf16 combine" if fp8 else {"bfloat16": "bf16", "float16": "f16"}[
-            str(cfg.in_dtype).replace("torch.", "")],
-        data="synthetic",
-        config=dict(workload=args.workload, tokens=T, experts=E, top_k=K, hidden=H, emulated_ranks=W,
-                    routed_rows=T * K, combine=args.combine, launch="hipGraph replay, two steps per graph" if use_graph else "eager",
-                    fused_route=bool(not args.no_fuse_route and not fp8 and lib.moe_a2a_fused_ok(T, K, H)),
-                    fused_stub=bool(args.fuse_stub)),
-        dispatch_combine_us=round(t_dc, 3), route_us=round(t_route, 3), dispatch_us=round(t_disp, 3),
-        stub_us=round(t_stub, 3), combine_us=round(t_comb, 3),
+        metric=METRIC, value=round(value, 1), unit="GB/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
+        ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None, dtype=dtype,
+        data="synthetic", config=config,
+        dispatch_combine_us=round(t["dc"], 3), route_us=round(t["route"], 3), dispatch_us=round(t["dispatch"], 3),
+        stub_us=round(t["stub"], 3), combine_us=round(t["combine"], 3),
         pct_of_hbm_peak=round(100.0 * value / HBM_PEAK_GBPS, 2),
-        tokens_per_s=round(T / (t_dc * 1e-6), 1),
+        tokens_per_s=round(T / (t["dc"] * 1e-6), 1),
         tokens_per_s_wall=round(T / (ms_per_step * 1e-3), 1),
-        eager_ms_per_step=round(eager_ms_per_step, 6),
-        timed_passes=dict(wall_us_per_step=round(pass_wall[0], 3), plain_lead_passes=lead,
-                          host_us_per_plain_pass=round(host_plain_us, 2), host_us_per_timed_pass=round(host_timed_us, 2)),
+        eager_ms_per_step=round(det["eager_ms_per_step"], 6),
+        timed_passes={k: v for k, v in det.items() if k != "eager_ms_per_step"},
         bytes=dict(dispatch=ab["dispatch"], combine=ab["combine"], stub=ab["stub"]),
         kernels=summarise(per),
         roofline=roofline,
     )
 
-    if mode == contract.COMBINE_STRICT and not args.fuse_stub:
-        # The same step with the f32-accumulating combine (one rounding at the end; within the
-        # rtol = atol = 1e-2 bar instead of bit-identical to the reference's per-step rounding):
-        # reported beside the headline value, never in place of it.
-        ata32 = HipAllToAll(cfg, 0, W, stub_kind=wl.stub_kind, combine_mode=contract.COMBINE_F32, fp8_dispatch=fp8,
-                            fuse_route=not args.no_fuse_route)
-        with torch.cuda.stream(main):
-            step32 = ata32.plan(x, idx, w, rs, stream=main)
-            step32()
-            step32()
-            main.synchronize()
-            run32 = c_loop(step32)
-            run32(4)
-            main.synchronize()
-            per32 = kernel_times(lib, run32, args.steps, torch, lead=lead, launches_per_step=n_launch)
-        t32 = (per_step(per32, ROUTE_KERNELS, args.steps) + per_step(per32, DISPATCH_KERNELS, args.steps) +
-               per_step(per32, COMBINE_KERNELS, args.steps))
-        out["f32_combine"] = dict(dispatch_combine_us=round(t32, 3),
-                                  combine_us=round(per_step(per32, COMBINE_KERNELS, args.steps), 3),
-                                  value=round(b_dc / t32 / 1e3, 1),
-                                  pct_of_hbm_peak=round(100.0 * b_dc / t32 / 1e3 / HBM_PEAK_GBPS, 2))
+    if not args.single:
+        # The same path with the expert stand-in as a launch of its own (three launches per step; the
+        # stub's time is then outside dispatch+combine) ...
+        other = Leg(torch, lib, wl, tensors, main, mode, fp8, fuse_route, not fuse_stub)
+        o_ms = other.graph_wall(args.steps, args.warmup, use_graph)
+        o_per, _ = other.kernels(args.steps, args.warmup, o_ms * 1e3)
+        ot = phase_times(o_per, args.steps)
+        out["stub_folded_into_combine" if not fuse_stub else "stub_as_its_own_launch"] = dict(
+            dispatch_combine_us=round(ot["dc"], 3), dispatch_us=round(ot["dispatch"] + ot["route"], 3),
+            stub_us=round(ot["stub"], 3), combine_us=round(ot["combine"], 3), ms_per_step=round(o_ms, 6),
+            value=round(b_dc / ot["dc"] / 1e3, 1), pct_of_hbm_peak=round(100.0 * b_dc / ot["dc"] / 1e3 / HBM_PEAK_GBPS, 2))
+        del other
+        if mode == contract.COMBINE_STRICT:
+            # ... and with the f32-accumulating combine (one rounding at the end; within the
+            # rtol = atol = 1e-2 bar instead of bit-identical to the reference's per-step rounding):
+            # reported beside the headline value, never in place of it.
+            l32 = Leg(torch, lib, wl, tensors, main, contract.COMBINE_F32, fp8, fuse_route, fuse_stub)
+            p32, _ = l32.kernels(args.steps, args.warmup, ms_per_step * 1e3)
+            t32 = phase_times(p32, args.steps)
+            out["f32_combine"] = dict(dispatch_combine_us=round(t32["dc"], 3), combine_us=round(t32["combine"], 3),
+                                      value=round(b_dc / t32["dc"] / 1e3, 1),
+                                      pct_of_hbm_peak=round(100.0 * b_dc / t32["dc"] / 1e3 / HBM_PEAK_GBPS, 2))
+            del l32
 
     if args.cold:
         # cold caches: overwrite 1 GiB (4x the 256 MB Infinity Cache) before every step
         flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         n_cold = min(args.steps, 30)
-
         with torch.cuda.stream(main):
             flush.fill_(1)
-            run_n(2)
-            perc = kernel_times(lib, run_n, n_cold, torch, before_each=lambda: flush.fill_(1))
+            leg.run_n(2)
+            perc = kernel_times(lib, leg.run_n, n_cold, torch, before_each=lambda: flush.fill_(1))
         tc = per_step(perc, ROUTE_KERNELS + DISPATCH_KERNELS + COMBINE_KERNELS, n_cold)
         out["cold"] = dict(dispatch_combine_us=round(tc, 3), GBps=round(b_dc / tc / 1e3, 1),
                            pct_of_hbm_peak=round(100.0 * b_dc / tc / 1e3 / HBM_PEAK_GBPS, 2),
@@ -362,17 +462,87 @@ def main():
         del flush
 
     if args.calibrate_copy:
-        with torch.cuda.stream(main):
-            src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
-            dst = torch.empty_like(src)
-            for _ in range(3):
-                dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibrate_copy(torch, main, dev)
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(wl, mode, fp8, y, b_dc, args.cpu_seconds)
+        out["cpu_baseline"] = cpu_baseline(wl, mode, fp8, leg.y, b_dc, args.cpu_seconds)
     print(json.dumps(out, ensure_ascii=False), flush=True)
+
+
+def calibrate_copy(torch, main, dev):
+    """Three plain 256 MiB device copies: the known-size reference for the profiler's byte counters."""
+    with torch.cuda.stream(main):
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+    torch.cuda.synchronize()
+
+
+KERNEL_OF_SYMBOL = (("route_dispatch_tile_kernel", "route_dispatch_tile"), ("route_dispatch_kernel", "route_dispatch"),
+                    ("stub_combine_rows_kernel", "stub_combine"), ("stub_combine_fp8_kernel", "stub_combine"),
+                    ("combine_rows_kernel", "combine_rows"), ("dispatch_rows_kernel", "dispatch_rows"),
+                    ("dispatch_fp8_kernel", "dispatch_fp8"), ("stub_rows_kernel", "stub_rows"),
+                    ("stub_fp8_kernel", "stub_fp8"))
+
+
+def record_traffic(directory):
+    """Fold the counter CSVs of `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of
+    `bench.py --graph-only --calibrate-copy --workload W` into profiles/traffic.json.
+
+    `directory` holds one sub-directory per run named <workload>_<COUNTER> with rocprofv3's
+    *_counter_collection.csv inside.  The scale of each counter is what it reads for the 256 MiB
+    copies at the end of every run.  Each entry records the kernel's symbol, the hash of the kernel
+    sources and the commit the tree was at."""
+    import csv
+    import glob
+    import subprocess
+
+    COPY_BYTES = 256 << 20
+    runs = {}
+    for path in sorted(glob.glob(os.path.join(directory, "*", "**", "*counter_collection.csv"), recursive=True)):
+        run = os.path.relpath(path, directory).split(os.sep)[0]
+        workload, counter = run.rsplit("_", 2)[0], "_".join(run.rsplit("_", 2)[1:])
+        per_kernel = {}
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] != counter:
+                    continue
+                per_kernel.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        runs[(workload, counter)] = per_kernel
+    if not runs:
+        raise SystemExit(f"no *_counter_collection.csv under {directory}/<workload>_<COUNTER>/")
+    try:
+        commit = subprocess.run(["git", "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True,
+                                cwd=ROOT).stdout.strip() or "?"
+    except OSError:
+        commit = "?"
+    factor, entries, src = {}, [], kernel_source_hash()
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        reads = [statistics.median(v) for (wl_, c), ks in runs.items() if c == counter
+                 for k, v in ks.items() if "copyBuffer" in k]
+        if not reads:
+            raise SystemExit(f"no calibration copy in the {counter} runs (run bench.py with --calibrate-copy)")
+        factor[counter] = round(COPY_BYTES / (statistics.median(reads) * 1024.0), 3)
+    for workload in sorted({wl_ for wl_, _ in runs}):
+        fetch, write = runs.get((workload, "FETCH_SIZE"), {}), runs.get((workload, "WRITE_SIZE"), {})
+        for symbol in sorted(set(fetch) & set(write)):
+            name = next((n for pat, n in KERNEL_OF_SYMBOL if pat in symbol), None)
+            if name is None:
+                continue
+            f_kib, w_kib = statistics.median(fetch[symbol]), statistics.median(write[symbol])
+            entries.append(dict(workload=workload, kernel=name, symbol=symbol.split("(")[0][:120],
+                                fetch_kib=round(f_kib, 1), write_kib=round(w_kib, 1),
+                                bytes=int((f_kib * factor["FETCH_SIZE"] + w_kib * factor["WRITE_SIZE"]) * 1024),
+                                launches=len(fetch[symbol]), source_hash=src, commit=commit))
+    rec = dict(what="HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, L2 <-> fabric), "
+                    "median over the launches of `bench.py --graph-only --calibrate-copy --workload W`",
+               factor=factor, factor_from="the same counters' medians for the three 256 MiB device copies that end each run",
+               entries=entries)
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    print(f"wrote {TRAFFIC_FILE}: {len(entries)} entries, factors {factor}, sources {src}, commit {commit}")
 
 
 MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16

@@ -14,9 +14,10 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer into caller-owned memory unless marked host;
- *   - the library allocates nothing, never synchronises and keeps no mutable state
- *     besides the opt-in launch timer at the end of this file; every launch goes to
- *     the stream passed in, so a call sequence can be captured into a hipGraph;
+ *   - the library allocates nothing, never synchronises, reads no environment variable and
+ *     keeps no mutable state besides the opt-in launch timer and the option switches at the
+ *     end of this file (both off unless the caller turns them on); every launch goes to the
+ *     stream passed in, so a call sequence can be captured into a hipGraph;
  *   - return value: 0 success, < 0 argument error found on the host before any
  *     launch (MOE_A2A_E_*), > 0 a hipError_t reported by the launch.
  */
@@ -30,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MOE_A2A_ABI_VERSION 3
+#define MOE_A2A_ABI_VERSION 4
 
 /* element types of activations */
 #define MOE_A2A_F16 0
@@ -53,6 +54,11 @@ extern "C" {
 /* scale of an fp8 block: amax / 448 in f32, or that rounded up to a power of two */
 #define MOE_A2A_FP8_SCALE_F32 0
 #define MOE_A2A_FP8_SCALE_POW2 1
+
+/* bits of the status word the routing entry points write (OR-ed into what the word holds, so the
+ * caller clears it; a call that meets both conditions reports both) */
+#define MOE_A2A_STATUS_BAD_EXPERT 1 /* an expert id was outside [0, E) and has been clamped      */
+#define MOE_A2A_STATUS_OVERFLOW 2   /* padded layout: an expert has more than max_recv entries   */
 
 /* argument errors */
 #define MOE_A2A_E_NULL (-1)      /* a required pointer is NULL                       */
@@ -86,8 +92,9 @@ size_t moe_a2a_workspace_bytes(int T, int K, int E);
  *   src_of_slot[R]       row -> entry (inverse permutation)
  *   meta[R,5]            per row: [e, source rank, token within its rank, k, 0]
  *                        (all2all/reference.py:85)
- *   status               optional int32[1]: set to 1 if an expert id was out of range
- *                        (such ids are clamped into [0,E) so no access goes out of bounds)
+ *   status               optional int32[1], cleared by the caller: MOE_A2A_STATUS_BAD_EXPERT is
+ *                        OR-ed in if an expert id was out of range (such ids are clamped into
+ *                        [0,E) so no access goes out of bounds), MOE_A2A_STATUS_OVERFLOW as below
  *   max_recv             0: compact layout, rows of all experts back to back (R rows).
  *                        > 0: the reference's padded layout (all2all/reference.py:65,127-136):
  *                        expert e owns rows [e*max_recv, (e+1)*max_recv), its j-th entry sits at
@@ -95,8 +102,11 @@ size_t moe_a2a_workspace_bytes(int T, int K, int E);
  *                        viewed as [W, E_l, max_recv, .], are the expert_x / expert_meta of every
  *                        owner rank; rows past counts[e] are not written.  slot_of_entry then
  *                        holds these physical rows, which is all dispatch and combine follow.
- *                        An expert with more than max_recv entries sets status to 2 (the extra
- *                        entries are folded onto the segment's last row).
+ *                        An expert with more than max_recv entries raises MOE_A2A_STATUS_OVERFLOW
+ *                        (the extra entries are folded onto the segment's last row; counts stay
+ *                        the true numbers).
+ * T == 0 (indices may then be NULL): counts and offsets are written as zeros by a kernel that is
+ * never handed the routing table; nothing else is written.
  */
 int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
                   int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
@@ -110,6 +120,13 @@ int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_ran
  */
 int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, int T, int K, int H,
                      moe_a2a_stream_t stream);
+
+/*
+ * Name of the kernel moe_a2a_route launches first for T tokens of top-K ("route_empty",
+ * "route_tiles" or "route_hist"): host logic only, usable without a GPU (the reference has no
+ * counterpart; a caller sizing its workspace, or a test, asks which form a shape takes).
+ */
+const char* moe_a2a_route_plan(int T, int K);
 
 /*
  * Routing and dispatch in ONE launch: every workgroup derives the slots of its own tokens from
@@ -200,7 +217,9 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
  *   Kd % 64 == 0, N % 8 == 0, 16-byte aligned.
  * Three kernels with identical results: 128 x 128 output tiles; 256 x 256 tiles when segments are
  * long (R >= 256 * E and N >= 256); 32 x 128 tiles that stream the weights when segments are short
- * (R <= 32 * E and Kd % 128 == 0).  MOE_A2A_GEMM_TILE=32, 128 or 256 in the environment forces one.
+ * (R <= 32 * E and Kd % 128 == 0).  The option MOE_A2A_OPT_GEMM_TILE = 32, 128 or 256 forces one.
+ * Padded layout: a segment longer than max_recv (routing raised MOE_A2A_STATUS_OVERFLOW) is
+ * multiplied over its first max_recv rows only, so no tile leaves the segment or the buffers.
  */
 int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offsets, void* y, int R, int E, int Kd,
                         int N, int max_recv, int elem_type, moe_a2a_stream_t stream);
@@ -229,7 +248,7 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
  *     cores exactly (turned into 16-bit values in registers), each 128-wide K block is summed in
  *     f32 and scaled in f32: y = sum over K blocks of scale_b * (x . q_b).  fp8 rows: the bytes of
  *     both operands go to the fp8 matrix instruction untouched, folded per K block as below.
- *     MOE_A2A_Q8_STREAM=0 / MOE_A2A_F8_STREAM=0 select the register-staged form of the same
+ *     The option MOE_A2A_OPT_GEMM_STAGED = 1 selects the register-staged form of the same
  *     arithmetic (fp8 rows are then dequantised and rounded once to elem_type first).
  *   longer segments, fp8 rows: both operands enter the fp8 matrix instruction as bytes
  *     (v_mfma_f32_32x32x64_f8f6f4), each 128-wide K block is summed in f32 and folded with
@@ -238,8 +257,8 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
  *     cores as elem(f32(q) * scale), i.e. dequantised and rounded once to elem_type on its way into
  *     LDS -- the result of dequantising the weights to 16 bits and calling moe_a2a_expert_gemm,
  *     without the 16-bit copy in memory.
- * The three differ by those roundings (2^-9 relative per operand for bf16); MOE_A2A_GEMM_TILE=32,
- * 128 (fp8 rows) or 256 forces one.  No counterpart in the reference.
+ * The three differ by those roundings (2^-9 relative per operand for bf16); the option
+ * MOE_A2A_OPT_GEMM_TILE = 32, 128 (fp8 rows) or 256 forces one.  No counterpart in the reference.
  */
 int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
@@ -256,8 +275,9 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
  * x_scale * w_scale * (q_x . q_w) in f32, one rounding to elem_type.  ONLY the exponent field of a
  * scale is used: a scale that is not a power of two is silently taken as the power of two below
  * it.  Segments of at most 32 rows on average (a decode step), and other Kd on segments shorter
- * than 256 rows, go through moe_a2a_expert_gemm_q8 (any f32 scale).  MOE_A2A_GEMM_TILE=256 forces
- * the tiles, 32 / 128 the kernels of moe_a2a_expert_gemm_q8.  Arguments as for
+ * than 256 rows, go through moe_a2a_expert_gemm_q8 (any f32 scale).  The option
+ * MOE_A2A_OPT_GEMM_TILE = 256 forces the tiles, 32 / 128 the kernels of moe_a2a_expert_gemm_q8,
+ * MOE_A2A_OPT_GEMM_STAGED = 1 the register-staged loop of the tiles.  Arguments as for
  * moe_a2a_expert_gemm_q8 with x_scale required.  No counterpart in the reference.
  */
 int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w_q, const float* w_scale,
@@ -280,6 +300,24 @@ int moe_a2a_timer_begin(int capacity);
 int moe_a2a_timer_skip(int launches);
 int moe_a2a_timer_end(int* kernel_ids, float* microseconds, int n);
 const char* moe_a2a_kernel_name(int kernel_id);
+
+/*
+ * Option switches (opt-in, process-wide; every option starts at 0 = the library decides).  They
+ * force one of several kernels that give the same results, for tests that compare the kernels with
+ * each other and for measurements; they are plain integers read at launch time, so a caller that
+ * never sets one pays nothing and sees no hidden behaviour.
+ *   set_option(option, value)  returns the previous value, or MOE_A2A_E_DTYPE for an unknown option
+ *   get_option(option)         current value, or MOE_A2A_E_DTYPE
+ */
+#define MOE_A2A_OPT_ROUTE_TILE 0    /* 1: moe_a2a_route_dispatch takes the token-tile kernel at any size   */
+#define MOE_A2A_OPT_GEMM_TILE 1     /* 32 | 128 | 256: tile family of the expert GEMM entry points          */
+#define MOE_A2A_OPT_GEMM_STAGED 2   /* 1: register-staged form of the weight-streaming / scaled-MFMA loops  */
+#define MOE_A2A_OPT_COMBINE_LANES 3 /* lanes of a combine workgroup at cache-resident sizes (64 .. 512)     */
+#define MOE_A2A_OPT_COMBINE_VPL 4   /* 2: two row vectors per lane in the combine at cache-resident sizes   */
+#define MOE_A2A_OPT_TIMER_EVENT_FLAGS 5 /* hipEventCreateWithFlags value for the launch timer's events    */
+#define MOE_A2A_OPT_COUNT 6
+int moe_a2a_set_option(int option, int value);
+int moe_a2a_get_option(int option);
 
 #ifdef __cplusplus
 }

@@ -9,9 +9,12 @@ import os
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmoe_a2a.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 F16, BF16 = 0, 1
 FP8_SCALE_F32, FP8_SCALE_POW2 = 0, 1
+STATUS_BAD_EXPERT, STATUS_OVERFLOW = 1, 2  # bits of the routing status word
+# option switches of moe_a2a_set_option (0 = the library decides)
+OPT_ROUTE_TILE, OPT_GEMM_TILE, OPT_GEMM_STAGED, OPT_COMBINE_LANES, OPT_COMBINE_VPL, OPT_TIMER_EVENT_FLAGS = range(6)
 
 _i32p = C.c_void_p  # device pointers travel as plain addresses
 _vp = C.c_void_p
@@ -40,6 +43,9 @@ PROTOTYPES = {
     "moe_a2a_expert_gemm_fp8": (_int, [_vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_expert_gemm_q8": (_int, [_vp, _vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_expert_gemm_mx8": (_int, [_vp, _vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
+    "moe_a2a_route_plan": (C.c_char_p, [_int, _int]),
+    "moe_a2a_set_option": (_int, [_int, _int]),
+    "moe_a2a_get_option": (_int, [_int]),
     "moe_a2a_timer_begin": (_int, [_int]),
     "moe_a2a_timer_skip": (_int, [_int]),
     "moe_a2a_timer_end": (_int, [C.POINTER(C.c_int), C.POINTER(C.c_float), _int]),

@@ -60,12 +60,13 @@ enum KernelId {
   KID_EXPERT_GEMM_SKINNY,
   KID_EXPERT_GEMM_F8,
   KID_EXPERT_GEMM_MX,
+  KID_ROUTE_EMPTY,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
-    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx"};
+    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -112,9 +113,13 @@ __device__ __forceinline__ void unpack8(const uint4& v, uint32_t (&d)[4]) {
   d[3] = v.w;
 }
 
+// (1 + e) / E as the f32 nearest the exact quotient.  The oracle divides in double and rounds the
+// result to f32; for integers up to 1024 the correctly rounded f32 division gives the same value (a
+// quotient of such integers is never within 2^-53 relative of an f32 rounding boundary without lying
+// on it), at a quarter of the instructions.
 __device__ __forceinline__ float stub_factor(int e, int stub_kind, int num_experts, int experts_per_rank) {
   if (stub_kind == MOE_A2A_STUB_OWNER_RANK) return (float)(1 + e / experts_per_rank);
-  return (float)((double)(1 + e) / (double)num_experts);
+  return __fdiv_rn((float)(1 + e), (float)num_experts);
 }
 
 // the kernels, in three files of their own
@@ -189,26 +194,80 @@ RowGeom row_geom(int nvec, int unit = 1, int max_threads = kRowMaxThreads, int m
   return g;
 }
 
+// Geometry of the combine kernels: `per` lanes of a workgroup hold `vpl` row vectors each.
+struct CombineGeom {
+  int per, nsplit, threads, vpl;
+};
+// Dynamic LDS beyond the 48 KB default needs the function's attribute raised.  The attribute belongs
+// to a device's copy of the function, so the largest size granted so far is kept per kernel and
+// device and the runtime is only asked when a launch needs more (racing first calls repeat it).
+template <auto Kernel>
+int ensure_lds(size_t bytes) {
+  if (bytes <= 48 * 1024) return 0;
+  static std::atomic<size_t> granted[kMaxDevices];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return MOE_A2A_E_STATE;
+  if (granted[dev].load(std::memory_order_acquire) >= bytes) return 0;
+  if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      e != hipSuccess)
+    return (int)e;
+  granted[dev].store(bytes, std::memory_order_release);
+  return 0;
+}
+
+// Process-wide switches of moe_a2a_set_option; 0 = automatic.
+std::atomic<int> g_option[MOE_A2A_OPT_COUNT];
+inline int option(int which) { return g_option[which].load(std::memory_order_relaxed); }
+
 // Combine at cache-resident sizes: about four workgroups per CU (1024 in all) finish sooner than
 // fewer, wider ones (256 tokens of 896 vectors: 4 x 224 lanes 6.4 us, 2 x 448 lanes 6.7 us); a
 // workgroup keeps at least 128 lanes.  Streaming sizes keep the widest workgroups (512 lanes).
-RowGeom combine_geom_resident(int nvec, int T) {
-  int nsplit = ceil_div(1024, T > 0 ? T : 1);
-  if (nsplit > nvec / 128) nsplit = nvec / 128;
-  const int least = ceil_div(nvec, kRowMaxThreads);
-  if (nsplit < least) nsplit = least;
-  RowGeom g;
-  g.nsplit = nsplit;
-  g.per = ceil_div(nvec, nsplit);
+// MOE_A2A_OPT_COMBINE_LANES / _VPL override both (measurements).
+CombineGeom combine_geom(int nvec, int T, bool streaming) {
+  CombineGeom g;
+  g.vpl = 1;
+  if (const int lanes = option(MOE_A2A_OPT_COMBINE_LANES)) {
+    g.vpl = option(MOE_A2A_OPT_COMBINE_VPL) == 2 && !streaming ? 2 : 1;
+    g.per = std::min(std::max(lanes, 1), kRowMaxThreads);
+    g.nsplit = ceil_div(nvec, g.per * g.vpl);
+  } else if (streaming) {
+    const RowGeom r = row_geom(nvec);
+    g.per = r.per;
+    g.nsplit = r.nsplit;
+  } else {
+    int nsplit = ceil_div(1024, T > 0 ? T : 1);
+    if (nsplit > nvec / 128) nsplit = nvec / 128;
+    const int least = ceil_div(nvec, kRowMaxThreads);
+    if (nsplit < least) nsplit = least;
+    g.nsplit = nsplit;
+    g.per = ceil_div(nvec, nsplit);
+  }
   g.threads = ceil_div(g.per, kWave) * kWave;
   return g;
 }
 
-template <typename F>
-void set_max_lds(F kernel, size_t bytes) {
-  if (bytes > 48 * 1024)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)bytes);
+// Routing of a table beyond kRouteTilesMaxRows entries: two launches (three beyond
+// kRouteFoldMaxTiles tiles) around the tile-major count matrix `tile` (ceil(R / 1024) x E ints).
+int route_large(const RouteArgs& a, int32_t* tile, hipStream_t stream) {
+  const size_t lds_w = (size_t)kRouteWaves * a.E * sizeof(int);
+  const size_t lds_starts = (size_t)(a.W + 1) * sizeof(int);
+  const int ntiles = ceil_div(a.R, kRouteThreads);
+  if (int rc = ensure_lds<route_hist_kernel>(lds_w)) return rc;
+  if (int rc = launch(KID_ROUTE_HIST, route_hist_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w, stream, a, tile))
+    return rc;
+  if (ntiles <= kRouteFoldMaxTiles) {  // scan folded into the rank launch
+    if (int rc = ensure_lds<route_rank_fold_kernel>(lds_w + lds_starts)) return rc;
+    return launch(KID_ROUTE_RANK, route_rank_fold_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w + lds_starts,
+                  stream, a, (const int32_t*)tile, ntiles);
+  }
+  if (int rc = launch(KID_ROUTE_SCAN, route_scan_kernel, dim3(1), dim3(kRouteThreads), 0, stream, tile, a.E, ntiles,
+                      a.counts, a.offsets))
+    return rc;
+  if (int rc = ensure_lds<route_rank_kernel>(lds_w + lds_starts)) return rc;
+  return launch(KID_ROUTE_RANK, route_rank_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w + lds_starts, stream, a,
+                (const int32_t*)tile);
 }
 
 }  // namespace
@@ -240,6 +299,13 @@ size_t moe_a2a_workspace_bytes(int T, int K, int E) {
   return align_up((size_t)ntiles * (size_t)E * sizeof(int32_t), 256);
 }
 
+// Which kernel moe_a2a_route launches first for this shape (host logic only, no GPU needed).
+static int route_first_kernel(int T, int K) {
+  const long long R = (long long)T * K;
+  if (R == 0) return KID_ROUTE_EMPTY;
+  return R <= kRouteTilesMaxRows ? KID_ROUTE_TILES : KID_ROUTE_HIST;
+}
+
 int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
                   int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
                   int32_t* meta, int32_t* status, void* workspace, size_t workspace_bytes,
@@ -249,33 +315,22 @@ int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_ran
   if (!counts || !offsets) return MOE_A2A_E_NULL;
   if (T > 0 && (!indices || !slot_of_entry || !src_of_slot || !meta)) return MOE_A2A_E_NULL;
   hipStream_t stream = (hipStream_t)stream_;
+  // No token: counts and offsets are zero and nothing else is written.  A kernel of its own, which
+  // is never handed `indices` (NULL is allowed here), does that.
+  if (T == 0)
+    return launch(KID_ROUTE_EMPTY, route_empty_kernel, dim3(1), dim3(kRouteThreads), 0, stream, counts, offsets, E);
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
               slot_of_entry, src_of_slot, meta, status};
   const size_t lds_w = (size_t)kRouteWaves * E * sizeof(int);
   const size_t lds_starts = (size_t)(W + 1) * sizeof(int);
   if (a.R <= kRouteTilesMaxRows) {
     size_t lds = lds_w + 2 * (size_t)E * sizeof(int) + (kRouteWaves + 1) * sizeof(int) + lds_starts;
-    set_max_lds(route_tiles_kernel, lds);
-    return launch(KID_ROUTE_TILES, route_tiles_kernel, dim3(a.R ? ceil_div(a.R, kRouteThreads) : 1),
-                  dim3(kRouteThreads), lds, stream, a);
+    if (int rc = ensure_lds<route_tiles_kernel>(lds)) return rc;
+    return launch(KID_ROUTE_TILES, route_tiles_kernel, dim3(ceil_div(a.R, kRouteThreads)), dim3(kRouteThreads), lds,
+                  stream, a);
   }
   if (!workspace || workspace_bytes < moe_a2a_workspace_bytes(T, K, E)) return MOE_A2A_E_WORKSPACE;
-  int ntiles = ceil_div(a.R, kRouteThreads);
-  int32_t* tile = (int32_t*)workspace;
-  set_max_lds(route_hist_kernel, lds_w);
-  if (int rc = launch(KID_ROUTE_HIST, route_hist_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w, stream, a, tile))
-    return rc;
-  if (ntiles <= kRouteFoldMaxTiles) {  // scan folded into the rank launch
-    set_max_lds(route_rank_fold_kernel, lds_w + lds_starts);
-    return launch(KID_ROUTE_RANK, route_rank_fold_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w + lds_starts,
-                  stream, a, (const int32_t*)tile, ntiles);
-  }
-  if (int rc = launch(KID_ROUTE_SCAN, route_scan_kernel, dim3(1), dim3(kRouteThreads), 0, stream, tile, E, ntiles,
-                      counts, offsets))
-    return rc;
-  set_max_lds(route_rank_kernel, lds_w + lds_starts);
-  return launch(KID_ROUTE_RANK, route_rank_kernel, dim3(ntiles), dim3(kRouteThreads), lds_w + lds_starts, stream, a,
-                (const int32_t*)tile);
+  return route_large(a, (int32_t*)workspace, stream);
 }
 
 static int check_rows(const void* a, const void* b, int T, int K, int H, int mult) {
@@ -377,8 +432,7 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
               slot_of_entry, src_of_slot, meta, status};
   const int nvec = H / 8;
-  const char* force_tile = getenv("MOE_A2A_ROUTE_TILE");  // tuning aid: 1 forces the token-tile kernel
-  if (!fused_small_ok(T, K, H) || (force_tile && atoi(force_tile) == 1)) {  // token tiles: any table size
+  if (!fused_small_ok(T, K, H) || option(MOE_A2A_OPT_ROUTE_TILE) == 1) {  // token tiles: any table size
     if (T == 0) return moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets,
                                      slot_of_entry, src_of_slot, meta, status, nullptr, 0, stream_);
     if (K > kTileMaxOwn) return MOE_A2A_E_SHAPE;
@@ -524,18 +578,17 @@ static int combine_impl(const void* expert_y, const float* weights, const int32_
   const int nvec = H / 8;
   const bool st = streams((long long)T * K, T, H, 2, 2);
   const bool through = dispatched_bytes > (256ll << 20);
-  const RowGeom g = st ? row_geom(nvec) : combine_geom_resident(nvec, T);
+  const CombineGeom g = combine_geom(nvec, T, st);
   dim3 grid((unsigned)T * g.nsplit), block(g.threads);
-#define COMBINE_LAUNCH(EL, MD, KT)                                                                            \
-  {                                                                                                           \
-    if (st && through)                                                                                        \
-      return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 2>, grid, block, 0, stream,                  \
-                    (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit);   \
-    if (st)                                                                                                   \
-      return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 1>, grid, block, 0, stream,                  \
-                    (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit);   \
-    return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 0>, grid, block, 0, stream,                    \
-                  (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit);     \
+#define COMBINE_ARGS (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit
+#define COMBINE_LAUNCH(EL, MD, KT)                                                                             \
+  {                                                                                                            \
+    if (st && through)                                                                                         \
+      return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 2, 1>, grid, block, 0, stream, COMBINE_ARGS); \
+    if (st) return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 1, 1>, grid, block, 0, stream, COMBINE_ARGS); \
+    if (g.vpl == 2)                                                                                            \
+      return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 0, 2>, grid, block, 0, stream, COMBINE_ARGS); \
+    return launch(KID_COMBINE, combine_rows_kernel<EL, MD, KT, 0, 1>, grid, block, 0, stream, COMBINE_ARGS);   \
   }
 #define CALL_BS(KT) COMBINE_LAUNCH(Bf16, MOE_A2A_COMBINE_STRICT, KT)
 #define CALL_BF(KT) COMBINE_LAUNCH(Bf16, MOE_A2A_COMBINE_F32, KT)
@@ -553,6 +606,7 @@ static int combine_impl(const void* expert_y, const float* weights, const int32_
 #undef CALL_HS
 #undef CALL_HF
 #undef COMBINE_LAUNCH
+#undef COMBINE_ARGS
 }
 
 int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_t* indices, const float* weights,
@@ -600,17 +654,20 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
 #undef SC8_LAUNCH
   }
   const int nvec = H / 8;
-  const RowGeom g = st ? row_geom(nvec) : combine_geom_resident(nvec, T);
+  const CombineGeom g = combine_geom(nvec, T, st);
   dim3 grid((unsigned)T * g.nsplit), block(g.threads);
-#define SC_LAUNCH(IN, OUT, MD, KT)                                                                              \
-  {                                                                                                             \
-    if (st)                                                                                                     \
-      return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD, KT, 1>, grid, block, 0, stream,     \
-                    (const uint4*)disp, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K,     \
-                    nvec, g.per, g.nsplit);                                                                     \
-    return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD, KT, 0>, grid, block, 0, stream,       \
-                  (const uint4*)disp, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K, nvec, \
-                  g.per, g.nsplit);                                                                             \
+#define SC_ARGS \
+  (const uint4*)disp, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K, nvec, g.per, g.nsplit
+#define SC_LAUNCH(IN, OUT, MD, KT)                                                                            \
+  {                                                                                                           \
+    if (st)                                                                                                   \
+      return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD, KT, 1, 1>, grid, block, 0, stream, \
+                    SC_ARGS);                                                                                 \
+    if (g.vpl == 2)                                                                                           \
+      return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD, KT, 0, 2>, grid, block, 0, stream, \
+                    SC_ARGS);                                                                                 \
+    return launch(KID_STUB_COMBINE, stub_combine_rows_kernel<IN, OUT, MD, KT, 0, 1>, grid, block, 0, stream,  \
+                  SC_ARGS);                                                                                   \
   }
 #define CALL_BS(KT) SC_LAUNCH(Bf16, Bf16, MOE_A2A_COMBINE_STRICT, KT)
 #define CALL_BF(KT) SC_LAUNCH(Bf16, Bf16, MOE_A2A_COMBINE_F32, KT)
@@ -636,6 +693,7 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
 #undef CALL_HS
 #undef CALL_HF
 #undef SC_LAUNCH
+#undef SC_ARGS
 }
 #undef MOE_A2A_SWITCH_KT
 
@@ -735,20 +793,20 @@ int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offse
                         int N, int max_recv, int elem_type, moe_a2a_stream_t stream_) {
   if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
   if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < kGemmK || Kd % kGemmK != 0 || N < 8 || N % 8 != 0 ||
-      max_recv < 0)
+      max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8)
     return MOE_A2A_E_SHAPE;
   if (R == 0) return 0;
   if (!x || !weights || !offsets || !y) return MOE_A2A_E_NULL;
   if (!aligned16(x) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
   hipStream_t stream = (hipStream_t)stream_;
   // Long segments take the 256 x 256 kernel: with fewer than 256 rows per expert on average most
-  // of its tiles would be half empty.  MOE_A2A_GEMM_TILE=32|128|256 in the environment overrides.
+  // of its tiles would be half empty.  the option MOE_A2A_OPT_GEMM_TILE = 32 | 128 | 256 overrides.
   // Short segments (a decode step) take the 32 x 256 kernel, which streams the weights.
   bool wide = (long long)R >= 256ll * E && N >= kWideN;
   bool skinny = (long long)R <= 32ll * E;
-  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) {
-    wide = atoi(forced) == 256;
-    skinny = atoi(forced) == 32;
+  if (const int forced = option(MOE_A2A_OPT_GEMM_TILE)) {
+    wide = forced == 256;
+    skinny = forced == 32;
   }
   if (Kd % kSkinnyK != 0) skinny = false;  // its K slabs are 128 wide; the 128 x 128 kernel takes the rest
   if (wide) return launch_gemm_wide(x, nullptr, weights, nullptr, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
@@ -780,7 +838,7 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
                             moe_a2a_stream_t stream_) {
   if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
   if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 || N < 8 ||
-      N % 8 != 0 || max_recv < 0)
+      N % 8 != 0 || max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8)
     return MOE_A2A_E_SHAPE;
   if (R == 0) return 0;
   if (!x_q || !x_scale || !weights || !offsets || !y) return MOE_A2A_E_NULL;
@@ -794,7 +852,8 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
                            moe_a2a_stream_t stream_) {
   if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
   if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 ||
-      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0)
+      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0 ||
+      (long long)max_recv * E > (long long)INT32_MAX / 8)
     return MOE_A2A_E_SHAPE;
   if (R == 0) return 0;
   if (!x || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
@@ -802,13 +861,12 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
   hipStream_t stream = (hipStream_t)stream_;
   // A decode step streams the weights (32-row tiles); longer segments multiply fp8 by fp8 when the
   // rows are fp8, else on the 256 x 256 kernel, which dequantises the weights on their way into LDS
-  // (it needs N >= 256).  MOE_A2A_GEMM_TILE = 32 | 128 | 256 forces one where it applies.
+  // (it needs N >= 256).  The option MOE_A2A_OPT_GEMM_TILE = 32 | 128 | 256 forces one where it applies.
   enum { kStream, kBothFp8, kDequant } kernel;
   if ((long long)R <= 32ll * E) kernel = kStream;
   else if (x_scale) kernel = kBothFp8;
   else kernel = N >= kWideN ? kDequant : kStream;
-  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) {
-    const int tile = atoi(forced);
+  if (const int tile = option(MOE_A2A_OPT_GEMM_TILE)) {
     if (tile == 32) kernel = kStream;
     if (tile == 128 && x_scale) kernel = kBothFp8;
     if (tile == 256 && N >= kWideN) kernel = kDequant;
@@ -831,7 +889,7 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
     return launch(KID_EXPERT_GEMM_F8, expert_gemm_f8_kernel<F16, tn>, grid, block, 0, stream, (const uint4*)x,
                   x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
   }
-  if (x_scale && !(getenv("MOE_A2A_F8_STREAM") && atoi(getenv("MOE_A2A_F8_STREAM")) == 0)) {
+  if (x_scale && option(MOE_A2A_OPT_GEMM_STAGED) != 1) {
     // both operands fp8: the bytes stream memory -> LDS -> matrix cores, nothing is decoded
     const int ntile_n = N / kF8sN;
     const long long mtiles = (long long)R / kF8sM + E;
@@ -843,7 +901,7 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
     return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_f8s_kernel<F16>, grid, block, 0, stream, (const uint4*)x, x_scale,
                   (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
   }
-  if (!x_scale && !(getenv("MOE_A2A_Q8_STREAM") && atoi(getenv("MOE_A2A_Q8_STREAM")) == 0)) {
+  if (!x_scale && option(MOE_A2A_OPT_GEMM_STAGED) != 1) {
     // 16-bit rows: the slabs stream memory -> LDS, the weight bytes become 16-bit fragments in registers
     const int ntile_n = N / kF8sN;
     const long long mtiles = (long long)R / kF8sM + E;
@@ -877,7 +935,8 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
                             moe_a2a_stream_t stream_) {
   if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
   if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 ||
-      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0)
+      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0 ||
+      (long long)max_recv * E > (long long)INT32_MAX / 8)
     return MOE_A2A_E_SHAPE;
   if (R == 0) return 0;
   if (!x_q || !x_scale || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
@@ -888,15 +947,14 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
   // kernel that folds f32 scales on the vector units: 951 / 1140 us at 128 rows per expert,
   // 7168 -> 2048; 735 / 923 us and 2562 / 3420 us at 512 rows per expert, 4096 -> 2048 and -> 7168),
   // the register-staged loop for other Kd on long segments (3109 us in the last case), the folding
-  // kernel for what is left.  MOE_A2A_GEMM_TILE = 32 | 128 force the streaming / the folding kernel,
-  // 256 the tiles; MOE_A2A_MX_STAGED = 1 the register-staged loop.
+  // kernel for what is left.  The option MOE_A2A_OPT_GEMM_TILE = 32 | 128 forces the streaming / the folding kernel,
+  // 256 the tiles; MOE_A2A_OPT_GEMM_STAGED = 1 the register-staged loop.
   enum { kStream, kFold, kTilesDirect, kTilesStaged } kernel;
-  const bool staged_only = Kd % 256 != 0 || (getenv("MOE_A2A_MX_STAGED") && atoi(getenv("MOE_A2A_MX_STAGED")) == 1);
+  const bool staged_only = Kd % 256 != 0 || option(MOE_A2A_OPT_GEMM_STAGED) == 1;
   if ((long long)R <= 32ll * E) kernel = kStream;
   else if (!staged_only) kernel = kTilesDirect;
   else kernel = (long long)R >= 256ll * E ? kTilesStaged : kFold;
-  if (const char* forced = getenv("MOE_A2A_GEMM_TILE")) {
-    const int tile = atoi(forced);
+  if (const int tile = option(MOE_A2A_OPT_GEMM_TILE)) {
     if (tile == 32) kernel = kStream;
     if (tile == 128) kernel = kFold;
     if (tile == 256) kernel = staged_only ? kTilesStaged : kTilesDirect;
@@ -921,14 +979,30 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
                           (hipStream_t)stream_, true);
 }
 
+const char* moe_a2a_route_plan(int T, int K) {
+  if (T < 0 || K < 1) return "unknown";
+  return kKernelNames[route_first_kernel(T, K)];
+}
+
+int moe_a2a_set_option(int which, int value) {
+  if (which < 0 || which >= MOE_A2A_OPT_COUNT) return MOE_A2A_E_DTYPE;
+  return g_option[which].exchange(value, std::memory_order_relaxed);
+}
+
+int moe_a2a_get_option(int which) {
+  if (which < 0 || which >= MOE_A2A_OPT_COUNT) return MOE_A2A_E_DTYPE;
+  return option(which);
+}
+
 int moe_a2a_timer_begin(int capacity) {
   if (g_timer.active || capacity < 1) return MOE_A2A_E_STATE;
   g_timer.start = new hipEvent_t[capacity];
   g_timer.stop = new hipEvent_t[capacity];
   g_timer.ids = new int[capacity];
+  const unsigned flags = (unsigned)option(MOE_A2A_OPT_TIMER_EVENT_FLAGS);
   for (int i = 0; i < capacity; ++i) {
-    hipError_t e1 = hipEventCreate(&g_timer.start[i]);
-    hipError_t e2 = e1 == hipSuccess ? hipEventCreate(&g_timer.stop[i]) : e1;
+    hipError_t e1 = hipEventCreateWithFlags(&g_timer.start[i], flags);
+    hipError_t e2 = e1 == hipSuccess ? hipEventCreateWithFlags(&g_timer.stop[i], flags) : e1;
     if (e2 != hipSuccess) {  // give back what exists: events 0 .. i-1 in pairs, and start[i] if it was made
       if (e1 == hipSuccess) (void)hipEventDestroy(g_timer.start[i]);
       for (int j = 0; j < i; ++j) {

@@ -19,3 +19,31 @@ def gpu_device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+class _Options:
+    """Option switches of the library (moe_a2a_set_option) for one test; all back to 0 afterwards."""
+
+    def __init__(self):
+        from kernel_amd import _lib
+
+        self._lib_mod = _lib
+        self._lib = _lib.load()
+        self._touched = set()
+
+    def set(self, name, value):
+        opt = getattr(self._lib_mod, "OPT_" + name)
+        self._touched.add(opt)
+        rc = self._lib.moe_a2a_set_option(opt, int(value))
+        assert rc >= 0, rc
+
+    def reset(self):
+        for opt in self._touched:
+            self._lib.moe_a2a_set_option(opt, 0)
+
+
+@pytest.fixture
+def options():
+    o = _Options()
+    yield o
+    o.reset()

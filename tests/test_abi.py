@@ -154,6 +154,55 @@ def test_expert_gemm_rejects_bad_arguments(lib):
     assert gemm8(sc=None) == E_NULL
 
 
+def test_empty_world_never_reaches_a_kernel_that_reads_the_table(lib):
+    """T == 0 goes to the kernel that only writes zero counts and offsets; the kernels that read
+    `indices` are chosen for T >= 1 only.  (Host logic; the run on a GPU is in test_gpu_parity.py.)"""
+    assert lib.moe_a2a_route_plan(0, 8) == b"route_empty"
+    assert lib.moe_a2a_route_plan(0, 1) == b"route_empty"
+    assert lib.moe_a2a_route_plan(1, 1) == b"route_tiles"
+    assert lib.moe_a2a_route_plan(4096, 8) == b"route_tiles"
+    assert lib.moe_a2a_route_plan(4097, 8) == b"route_hist"
+    assert lib.moe_a2a_route_plan(-1, 8) == b"unknown"
+    assert lib.moe_a2a_fused_ok(0, 8, 7168) == 0  # and the one-launch forms are never picked for it
+    # T == 0 still needs somewhere to put the zeros, and takes NULL for everything else
+    assert lib.moe_a2a_route(None, None, 0, 0, 8, 256, 8, 0, None, A, None, None, None, None, None, 0, None) == E_NULL
+    assert lib.moe_a2a_route(None, None, 0, 0, 8, 256, 8, 0, A, None, None, None, None, None, None, 0, None) == E_NULL
+    # the other row entry points return before any launch
+    assert lib.moe_a2a_dispatch(None, None, None, 0, 8, 7168, None) == 0
+    assert lib.moe_a2a_combine(None, None, None, 0, _lib.BF16, None, 0, 8, 7168, None) == 0
+    assert lib.moe_a2a_stub_combine(None, None, None, None, None, 0, _lib.BF16, _lib.BF16, 0, 256, 8, None, 0, 8,
+                                    7168, None) == 0
+    assert lib.moe_a2a_stub(None, None, None, None, _lib.BF16, _lib.BF16, 0, 256, 8, None, 0, 7168, None) == 0
+
+
+def test_option_switches(lib):
+    for opt in range(6):
+        assert lib.moe_a2a_get_option(opt) == 0  # nothing is on unless a caller turns it on
+    assert lib.moe_a2a_set_option(_lib.OPT_GEMM_TILE, 128) == 0
+    assert lib.moe_a2a_get_option(_lib.OPT_GEMM_TILE) == 128
+    assert lib.moe_a2a_set_option(_lib.OPT_GEMM_TILE, 0) == 128  # returns the previous value
+    assert lib.moe_a2a_set_option(-1, 1) == E_DTYPE and lib.moe_a2a_set_option(6, 1) == E_DTYPE
+    assert lib.moe_a2a_get_option(99) == E_DTYPE
+
+
+def test_library_reads_no_environment_variable():
+    """The entry points take their switches from moe_a2a_set_option only."""
+    src = os.path.join(ROOT, "kernel_amd", "csrc")
+    for name in os.listdir(src):
+        if name.endswith((".hip", ".inc", ".cpp")):
+            assert "getenv" not in open(os.path.join(src, name)).read(), name
+
+
+def test_gemm_rejects_padded_buffers_beyond_the_addressable_rows(lib):
+    big = dict(E=1024, max_recv=1 << 20)
+    assert lib.moe_a2a_expert_gemm(A, A, A, A, 64, big["E"], 128, 64, big["max_recv"], _lib.BF16, None) == E_SHAPE
+    assert lib.moe_a2a_expert_gemm_fp8(A, A, A, A, A, 64, big["E"], 128, 64, big["max_recv"], _lib.BF16, None) == E_SHAPE
+    assert lib.moe_a2a_expert_gemm_q8(A, None, A, A, A, A, 64, big["E"], 128, 128, big["max_recv"], _lib.BF16,
+                                      None) == E_SHAPE
+    assert lib.moe_a2a_expert_gemm_mx8(A, A, A, A, A, A, 64, big["E"], 128, 128, big["max_recv"], _lib.BF16,
+                                       None) == E_SHAPE
+
+
 def test_timer_needs_begin_first(lib):
     ids = (ctypes.c_int * 4)()
     us = (ctypes.c_float * 4)()

@@ -153,3 +153,18 @@ def test_benchmark_and_profile_modes_on_the_gpu(gpu_device, tmp_path):
     report = [l for l in log.splitlines() if l.startswith("benchmark.0.report: ")][0].split(": ", 1)[1]
     text = base64.b64decode(report, b"+*").decode()
     assert "route_dispatch" in text and "stub_combine" in text  # custom_kernel folds the stub into the combine
+
+
+@pytest.mark.gpu
+def test_leaderboard_mode_on_the_gpu(gpu_device, tmp_path):
+    """`leaderboard` mode (eval.py:340-346, 369-372 of the reference): the inputs are generated anew
+    with seed + 13 for every repeat and EVERY run's output is checked, not only the first."""
+    f = tmp_path / "bench.txt"
+    f.write_text("\n".join(spec_line(s) for s in C.REFERENCE_BENCHMARKS[:2]))
+    code, log, err = run_cli(["leaderboard", str(f)], {"POPCORN_SEED": "99"})
+    assert code == 0, err + log
+    vals = dict(l.split(": ", 1) for l in log.splitlines())
+    assert vals["benchmark-count"] == "2" and vals["check"] == "pass"
+    for i in (0, 1):
+        assert int(vals[f"benchmark.{i}.runs"]) >= 3
+        assert float(vals[f"benchmark.{i}.best"]) <= float(vals[f"benchmark.{i}.mean"])

@@ -45,10 +45,10 @@ def make(E, K, T, H, N, W, dtype, seed, zipf=False):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
 @pytest.mark.parametrize("tile", ["32", "128", "256"], ids=["tile32", "tile128", "tile256"])
-def test_expert_gemm_matches_f32_reference(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, padded, tile):
+def test_expert_gemm_matches_f32_reference(gpu_device, options, E, K, T, H, N, W, zipf, dtype, padded, tile):
     # every kernel on every shape (the 32-row kernel needs H % 128 == 0; the library takes the
     # 128 x 128 kernel for the other hidden sizes)
-    monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile)
+    options.set("GEMM_TILE", tile)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=E + T, zipf=zipf)
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, W, padded=padded, max_recv=T if padded else None)
@@ -68,7 +68,7 @@ def test_expert_gemm_matches_f32_reference(gpu_device, monkeypatch, E, K, T, H, 
     (16, 4, 1500, 256, 512, True),   # skewed, segments from empty to well past one tile
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-def test_both_tile_sizes_give_the_same_bits(gpu_device, monkeypatch, E, K, T, H, N, zipf, dtype):
+def test_both_tile_sizes_give_the_same_bits(gpu_device, options, E, K, T, H, N, zipf, dtype):
     """The two kernels accumulate over K in the same order, so their outputs are identical; the
     default choice for these shapes (R >= 256 E) is the wide one."""
     cfg, world, weights = make(E, K, T, H, N, 1, dtype, seed=7 * E + T, zipf=zipf)
@@ -80,9 +80,9 @@ def test_both_tile_sizes_give_the_same_bits(gpu_device, monkeypatch, E, K, T, H,
     outs = {}
     for tile in ("default", "32", "128", "256"):
         if tile == "default":
-            monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
+            options.set("GEMM_TILE", 0)
         else:
-            monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile)
+            options.set("GEMM_TILE", tile)
         assert lib.moe_a2a_timer_begin(4) == 0
         outs[tile] = ata.expert_gemm(d, wd).clone()
         torch.cuda.synchronize()
@@ -138,10 +138,10 @@ def test_fp8_gemm_feeds_combine(gpu_device):
     close(y, want)
 
 
-def test_decode_shape_takes_the_skinny_kernel(gpu_device, monkeypatch):
+def test_decode_shape_takes_the_skinny_kernel(gpu_device, options):
     """Eight rows per expert on average (the headline routing shape): the library picks the
     32 x 256 kernel by itself, and its bits equal the 128 x 128 kernel's."""
-    monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
+    options.set("GEMM_TILE", 0)
     cfg, world, weights = make(256, 8, 256, 1024, 520, 8, torch.bfloat16, seed=11)
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, 8)
@@ -154,7 +154,7 @@ def test_decode_shape_takes_the_skinny_kernel(gpu_device, monkeypatch):
     ids, us = (ctypes.c_int * 4)(), (ctypes.c_float * 4)()
     assert ata.lib.moe_a2a_timer_end(ids, us, 4) == 1
     assert ata.lib.moe_a2a_kernel_name(ids[0]) == b"expert_gemm_skinny"
-    monkeypatch.setenv("MOE_A2A_GEMM_TILE", "128")
+    options.set("GEMM_TILE", "128")
     y128 = ata.expert_gemm(d, wd)
     assert torch.equal(y.view(torch.int16), y128.view(torch.int16))
     o = V.run_world(cfg, world)
@@ -171,7 +171,7 @@ def test_decode_shape_takes_the_skinny_kernel(gpu_device, monkeypatch):
 @pytest.mark.parametrize("fp8_rows", [False, True], ids=["rows16", "rows8"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
 @pytest.mark.parametrize("tile", ["32", "32r", "128", "256"], ids=["tile32", "tile32staged", "tile128", "tile256"])
-def test_expert_gemm_block_quantised_weights(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, fp8_rows,
+def test_expert_gemm_block_quantised_weights(gpu_device, options, E, K, T, H, N, W, zipf, dtype, fp8_rows,
                                              padded, tile):
     """Weights as e4m3fn bytes with one scale per 128 x 128 block, rows 16-bit or from the fp8
     dispatch, against an f32 matmul of the dequantised operands (each rounded once to the 16-bit
@@ -179,10 +179,9 @@ def test_expert_gemm_block_quantised_weights(gpu_device, monkeypatch, E, K, T, H
     128, fp8 rows only: 16-bit rows keep the default choice) and the 256 x 256 kernel (which needs
     N >= 256; the one N == 128 case stays on the other).  The weight-streaming form exists twice:
     slabs sent memory -> LDS directly (tile32) and staged through registers (tile32staged)."""
-    monkeypatch.setenv("MOE_A2A_GEMM_TILE", tile[:2] if tile.startswith("32") else tile)
+    options.set("GEMM_TILE", tile[:2] if tile.startswith("32") else tile)
     if tile == "32r":
-        monkeypatch.setenv("MOE_A2A_Q8_STREAM", "0")
-        monkeypatch.setenv("MOE_A2A_F8_STREAM", "0")
+        options.set("GEMM_STAGED", 1)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=5 * E + T, zipf=zipf)
     wq, ws = V.quantize_weights_fp8(weights)
     x, idx, w, rs = concat_world(world, gpu_device)
@@ -211,25 +210,25 @@ def test_expert_gemm_block_quantised_weights(gpu_device, monkeypatch, E, K, T, H
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
 @pytest.mark.parametrize("staged", [False, True], ids=["direct", "staged"])
-def test_expert_gemm_power_of_two_scales(gpu_device, monkeypatch, E, K, T, H, N, W, zipf, dtype, padded, staged):
+def test_expert_gemm_power_of_two_scales(gpu_device, options, E, K, T, H, N, W, zipf, dtype, padded, staged):
     """fp8 rows and fp8 weights whose scales are powers of two, multiplied by the fp8 matrix
     instruction with the scales as its block exponents, against the f32 matmul of the
     dequantised operands; the fp8 x fp8 kernel with the fold on the vector units, which takes
     any f32 scale, has to agree with it to f32 summation order.  Both forms of the tiled kernel:
     slabs sent memory -> LDS directly (hidden sizes that are multiples of 256) and staged through
     registers (every hidden size)."""
-    monkeypatch.setenv("MOE_A2A_GEMM_TILE", "256")  # the tiles at every segment length
+    options.set("GEMM_TILE", "256")  # the tiles at every segment length
     if staged:
-        monkeypatch.setenv("MOE_A2A_MX_STAGED", "1")
+        options.set("GEMM_STAGED", 1)
     else:
-        monkeypatch.delenv("MOE_A2A_MX_STAGED", raising=False)
+        options.set("GEMM_STAGED", 0)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=7 * E + T, zipf=zipf)
     wq, ws = V.quantize_weights_fp8(weights, pow2=True)
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, W, fp8_dispatch="pow2", padded=padded, max_recv=T if padded else None)
     d = ata.dispatch(x, idx, rs)
     y = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device), scales_pow2=True)
-    monkeypatch.delenv("MOE_A2A_GEMM_TILE")
+    options.set("GEMM_TILE", 0)
     y_auto = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device), scales_pow2=True)  # library's choice
     y_fold = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device))
     torch.cuda.synchronize()
@@ -239,6 +238,57 @@ def test_expert_gemm_power_of_two_scales(gpu_device, monkeypatch, E, K, T, H, N,
     close(y[rows], want[o["slot_of_entry"].long()])
     close(y[rows], y_fold[rows].cpu())
     close(y_auto[rows], want[o["slot_of_entry"].long()])
+
+
+@pytest.mark.parametrize("form", ["16bit-32", "16bit-128", "16bit-256", "q8-32", "q8-32staged", "q8-128", "q8-256",
+                                  "mx-direct", "mx-staged"])
+def test_padded_overflow_stays_inside_the_buffers(gpu_device, options, form):
+    """Padded layout with a LAST expert that receives more rows than max_recv (routing folds the
+    surplus onto the segment's last row and raises the overflow bit; counts stay the true numbers):
+    every GEMM form multiplies only the max_recv rows the segment holds.  Guard rows behind the
+    output keep their sentinel, the rows of the other experts and the unfolded rows of the full
+    expert equal the reference."""
+    from kernel_amd import _lib
+
+    E, K, T, H, N, W, max_recv = 8, 2, 300, 256, 256, 2, 96
+    dtype = torch.bfloat16
+    cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=11)
+    world[0].indices[:, 1] = E - 1  # every token also goes to the last expert: 300 rows for 96 places
+    world[0].indices[:, 0] %= E - 1
+    kind, tile = form.split("-")
+    options.set("GEMM_TILE", int(tile[:3].rstrip("sd")) if tile[0].isdigit() else 256)
+    if tile in ("32staged", "staged"):
+        options.set("GEMM_STAGED", 1)
+    fp8 = {"16bit": False, "q8": True, "mx": "pow2"}[kind]
+    x, idx, w, rs = concat_world(world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, fp8_dispatch=fp8, padded=True, max_recv=max_recv)
+    d = ata.dispatch(x, idx, rs)
+    rows = E * max_recv
+    guard = 2 * max_recv + 300  # more than the surplus of the overflowing expert
+    buf = torch.full((rows + guard, N), 7.0, dtype=dtype, device=gpu_device)
+    if kind == "16bit":
+        ata.expert_gemm(d, weights.to(gpu_device), out=buf[:rows])
+    else:
+        wq, ws = V.quantize_weights_fp8(weights, pow2=kind == "mx")
+        ata.expert_gemm(d, wq.to(gpu_device), out=buf[:rows], w_scale=ws.to(gpu_device), scales_pow2=kind == "mx")
+    torch.cuda.synchronize()
+    assert int(d.status.item()) == _lib.STATUS_OVERFLOW
+    assert int(d.counts[E - 1]) == T  # the true number, beyond the segment
+    assert bool((buf[rows:] == 7.0).all()), "rows behind the output buffer were written"
+    # reference: the same product on the rows the padded buffers hold
+    dx = d.disp_x.cpu()
+    sc = d.disp_scale.cpu() if fp8 else None
+    counts = d.counts.cpu().clamp(max=max_recv)
+    for e in range(E):
+        n = int(counts[e]) - (1 if e == E - 1 else 0)  # the folded entries race for the full segment's last row
+        lo = e * max_recv
+        seg = torch.tensor([0, n], dtype=torch.int32)
+        if kind == "16bit":
+            want = V.expert_gemm(dx[lo:lo + n], seg, weights[e:e + 1], dtype)
+        else:
+            want = V.expert_gemm_q8(dx[lo:lo + n], sc[lo:lo + n], wq[e:e + 1], ws[e:e + 1], seg, dtype,
+                                    round_rows=False)
+        close(buf[lo:lo + n], want)
 
 
 def test_dispatch_gemm_combine_end_to_end(gpu_device):
@@ -255,11 +305,11 @@ def test_dispatch_gemm_combine_end_to_end(gpu_device):
 
 
 @pytest.mark.parametrize("T,E", [(2048, 8), (96, 32)], ids=["wide", "skinny"])
-def test_dispatch_gemm_combine_graph_replay(gpu_device, monkeypatch, T, E):
+def test_dispatch_gemm_combine_graph_replay(gpu_device, options, T, E):
     """dispatch -> expert GEMM -> combine captured once into a hipGraph; every replay, with eager
     work and synchronisation between the replays and fresh inputs each time, equals the eager
     result bit for bit (no launch of the chain allocates, clears memory or reads a value back)."""
-    monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
+    options.set("GEMM_TILE", 0)
     cfg, world, weights = make(E, 2, T, 256, 256, 4, torch.bfloat16, seed=T)
     x, idx, w, rs = concat_world(world, gpu_device)
     wd = weights.to(gpu_device)
@@ -317,15 +367,15 @@ def test_expert_gemm_argument_checks(gpu_device):
 
 
 @pytest.mark.parametrize("seed", range(20))
-def test_random_shapes_every_expert_gemm_form(gpu_device, monkeypatch, seed):
+def test_random_shapes_every_expert_gemm_form(gpu_device, options, seed):
     """Seeded sweep: random expert counts, segment lengths (empty experts, segments that end a
     row or two past a tile), hidden and output sizes, layouts, element types, and every operand
     format (16-bit, fp8 rows, fp8 block-quantised weights, both) through whichever kernel the
     library picks for the shape and, on odd seeds, through a forced one."""
     g = torch.Generator().manual_seed(1000 + seed)
 
-    def pick(options):
-        return options[int(torch.randint(len(options), (1,), generator=g))]
+    def pick(choices):
+        return choices[int(torch.randint(len(choices), (1,), generator=g))]
 
     E = pick([1, 3, 8, 9, 24, 40])
     K = pick([1, 2, 4])
@@ -341,9 +391,9 @@ def test_random_shapes_every_expert_gemm_form(gpu_device, monkeypatch, seed):
     q8 = pick([False, True])
     pow2 = pick([False, True]) and fp8_rows and q8  # scales as the matrix instruction's block exponents
     if seed % 2:
-        monkeypatch.setenv("MOE_A2A_GEMM_TILE", pick(["32", "128", "256"]))
+        options.set("GEMM_TILE", pick(["32", "128", "256"]))
     else:
-        monkeypatch.delenv("MOE_A2A_GEMM_TILE", raising=False)
+        options.set("GEMM_TILE", 0)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=seed, zipf=zipf)
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, W, fp8_dispatch="pow2" if pow2 else fp8_rows, padded=padded,

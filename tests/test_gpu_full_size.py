@@ -211,3 +211,61 @@ def test_graph_replay_matches_eager(gpu_device):
     want_cpu = V.run_world(cfg, [C.RankData(T, nidx.cpu(), nw.cpu(), nx.cpu())] +
                            [C.RankData.empty(cfg) for _ in range(7)], stub_kind=wl.stub_kind)["y"]
     assert torch.equal(bits(y_static.cpu()), bits(want_cpu))
+
+
+@pytest.mark.parametrize("name,fuse_stub", [("prefill_graph", False), ("prefill_graph", True), ("fp8_dispatch", True)])
+def test_full_size_graph_replay_against_the_oracle(gpu_device, name, fuse_stub):
+    """The two streaming workloads at FULL size, the whole path captured once into a hipGraph: two
+    replays with eager work, a synchronisation and fresh inputs between them; the second replay's
+    dispatched rows, counts and output are compared bit for bit with the CPU oracle run on the same
+    inputs (the first with an eager run of the library)."""
+    wl = C.generate_workload(name)
+    cfg, W = wl.cfg, wl.world_size
+    fp8 = wl.fp8_dispatch
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    ata = HipAllToAll(cfg, 0, W, stub_kind=wl.stub_kind, fp8_dispatch=fp8, fuse_stub=fuse_stub)
+    sx, sidx, sw = x.clone(), idx.clone(), w.clone()  # static inputs of the graph
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ata.forward(sx, sidx, sw, rs)
+        ata.forward(sx, sidx, sw, rs)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_static = ata.forward(sx, sidx, sw, rs)
+    rec = ata.last
+    eager = HipAllToAll(cfg, 0, W, stub_kind=wl.stub_kind, fp8_dispatch=fp8, fuse_stub=fuse_stub)
+    T = x.shape[0]
+    # replay 1: the tokens in reverse order inside every rank's range stays a valid world only if whole
+    # ranks are kept, so the permutation moves tokens inside their rank
+    g = torch.Generator().manual_seed(5)
+    starts = rs.cpu().tolist()
+    perm = torch.cat([starts[r] + torch.randperm(starts[r + 1] - starts[r], generator=g) for r in range(W)])
+    permd = perm.to(gpu_device)
+    nx, nidx, nw = x[permd].contiguous(), idx[permd].contiguous(), w[permd].contiguous()
+    want = eager.forward(nx, nidx, nw, rs).clone()  # eager work between capture and replay
+    torch.cuda.synchronize()
+    sx.copy_(nx)
+    sidx.copy_(nidx)
+    sw.copy_(nw)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(bits(y_static), bits(want)), "replay 1 differs from the eager run"
+    # replay 2: the original inputs again, against the CPU oracle
+    eager.forward(x, idx, w, rs)
+    torch.cuda.synchronize()
+    sx.copy_(x)
+    sidx.copy_(idx)
+    sw.copy_(w)
+    graph.replay()
+    torch.cuda.synchronize()
+    o = V.run_world(cfg, wl.world, stub_kind=wl.stub_kind, fp8=bool(fp8))
+    assert torch.equal(rec.counts.cpu(), o["counts"]) and torch.equal(rec.slot_of_entry.cpu(), o["slot_of_entry"])
+    assert torch.equal(bits(rec.disp_x.cpu()), bits(o["disp_x"]))
+    if fp8:
+        assert torch.equal(rec.disp_scale.cpu(), o["disp_scale"])
+    assert torch.equal(bits(y_static.cpu()), bits(o["y"]))
+    ata.release_buffers()
+    eager.release_buffers()

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from golden_io import GOLDEN_CASES, bits, golden_compact, load_golden
-from kernel_amd import contract as C
+from kernel_amd import _lib, contract as C
 from kernel_amd.all2all import HipAllToAll, concat_world
 from oracle import all2all_vec as V
 
@@ -112,10 +112,10 @@ def test_multi_workgroup_routing(gpu_device):
 
 @pytest.mark.parametrize("name,scale", [("tiny", 1.0), ("dsv3_rank", 1.0), ("skew_world", 1.0), ("prefill_graph", 1 / 16)])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-def test_token_tile_kernel_on_every_size(gpu_device, monkeypatch, name, scale, padded):
+def test_token_tile_kernel_on_every_size(gpu_device, options, name, scale, padded):
     """The one-launch routing + dispatch with a tile of tokens per workgroup, forced for shapes the
     library would give to the one-token kernel or to separate launches: same bits everywhere."""
-    monkeypatch.setenv("MOE_A2A_ROUTE_TILE", "1")
+    options.set("ROUTE_TILE", 1)
     wl = C.generate_workload(name, tokens_scale=scale)
     cfg = wl.cfg
     x, idx, w, rs = concat_world(wl.world, gpu_device)
@@ -284,7 +284,7 @@ def _random_shapes(n, seed):
 
 
 @pytest.mark.parametrize("W,E,K,H,T,dup,seed", _random_shapes(24, 2024))
-def test_random_shapes_all_routing_kernels(gpu_device, monkeypatch, W, E, K, H, T, dup, seed):
+def test_random_shapes_all_routing_kernels(gpu_device, options, W, E, K, H, T, dup, seed):
     """Every routing implementation (one-token, token-tile, separate launches) on the same random
     world, compact and through the library's own choice: all bit-identical to the oracle."""
     g = torch.Generator().manual_seed(seed)
@@ -301,12 +301,12 @@ def test_random_shapes_all_routing_kernels(gpu_device, monkeypatch, W, E, K, H, 
             idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(n)]).to(torch.int32) if n else \
                 torch.empty(0, K, dtype=torch.int32)
         world.append(C.RankData(n, idx, torch.rand(n, K, generator=g), torch.randn(n, H, generator=g).to(torch.bfloat16)))
-    monkeypatch.delenv("MOE_A2A_ROUTE_TILE", raising=False)
+    options.set("ROUTE_TILE", 0)
     compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route=True)       # the library's choice
     compare(cfg, world, gpu_device, C.STUB_EXPERT_FRACTION, fuse_route=False)  # separate launches
-    monkeypatch.setenv("MOE_A2A_ROUTE_TILE", "1")
+    options.set("ROUTE_TILE", 1)
     compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route="always")   # token tiles
-    monkeypatch.setenv("MOE_A2A_ROUTE_TILE", "0")
+    options.set("ROUTE_TILE", 0)
     compare(cfg, world, gpu_device, C.STUB_OWNER_RANK, fuse_route="always")   # one-token kernel when it applies
 
 
@@ -422,11 +422,68 @@ def test_unaligned_index_slices_and_out_of_range_ids(gpu_device):
     clamped = bad.clamp(0, cfg.num_experts - 1)
     want = V.run_world(cfg, [C.RankData(T, clamped.cpu(), w.cpu(), x.cpu())], stub_kind=1)
     for fuse in ("always", False):
-        ata = HipAllToAll(cfg, 0, 1, stub_kind=1, fuse_route=fuse)
-        y = ata.forward(x, bad, w)
-        assert int(ata.last.status.item()) == 1
-        assert_same("slot_of_entry", ata.last.slot_of_entry, want["slot_of_entry"])
-        assert_same("disp_x", ata.last.disp_x, want["disp_x"])
+        for fuse_stub in (False, True):  # the folded stub takes its factor from the clamped id as well
+            ata = HipAllToAll(cfg, 0, 1, stub_kind=1, fuse_route=fuse, fuse_stub=fuse_stub)
+            y = ata.forward(x, bad, w)
+            assert int(ata.last.status.item()) == _lib.STATUS_BAD_EXPERT
+            assert_same("slot_of_entry", ata.last.slot_of_entry, want["slot_of_entry"])
+            assert_same("disp_x", ata.last.disp_x, want["disp_x"])
+            assert_same("y", y, want["y"])
+
+
+def test_status_reports_both_conditions(gpu_device):
+    """A call that meets an expert id out of range AND a padded segment that overflows reports both
+    bits, whichever lane gets there first; the word is sticky until the caller clears it."""
+    wl = C.generate_workload("skew_world")
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    bad = idx.clone()
+    bad[3, 0] = wl.cfg.num_experts + 5
+    bad[700, 2] = -1
+    for fuse_route in (False, "always"):
+        ata = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind, padded=True, max_recv=64,
+                          fuse_route=fuse_route)
+        ata.forward(x, bad, w, rs)
+        torch.cuda.synchronize()
+        assert int(ata.last.status.item()) == _lib.STATUS_BAD_EXPERT | _lib.STATUS_OVERFLOW
+        ata.last.status.zero_()
+        ata.forward(x, idx, w, rs)  # the other buffer set, clean ids: only the overflow is left
+        ata.forward(x, idx, w, rs)  # the first set again, after the caller cleared its word
+        torch.cuda.synchronize()
+        assert int(ata.last.status.item()) == _lib.STATUS_OVERFLOW
+
+
+def test_dispatch_of_an_empty_rank(gpu_device):
+    """No token at all: counts and offsets are zeros, nothing else is touched, and the routing
+    table (an empty tensor, whose address is not readable) is never read."""
+    cfg = C.MoEConfig(64, 6, 2048, 16, torch.bfloat16, torch.bfloat16)
+    x = torch.empty(0, cfg.hidden_dim, dtype=torch.bfloat16, device=gpu_device)
+    idx = torch.empty(0, cfg.experts_per_token, dtype=torch.int32, device=gpu_device)
+    w = torch.empty(0, cfg.experts_per_token, dtype=torch.float32, device=gpu_device)
+    for fuse_route in (True, False, "always"):
+        ata = HipAllToAll(cfg, 3, 8, fuse_route=fuse_route)
+        d = ata.dispatch(x, idx)
+        torch.cuda.synchronize()
+        assert d.num_rows == 0 and int(d.status.item()) == 0
+        assert torch.equal(d.counts.cpu(), torch.zeros(64, dtype=torch.int32))
+        assert torch.equal(d.offsets.cpu(), torch.zeros(65, dtype=torch.int32))
+        y = ata.combine(None, w, d, ata.expert_stub(d))
+        assert tuple(y.shape) == (0, cfg.hidden_dim)
+        assert tuple(ata.forward(x, idx, w).shape) == (0, cfg.hidden_dim)
+    # the same through the C entry points with NULL for everything that holds no element
+    lib = _lib.load()
+    counts = torch.full((64,), -1, dtype=torch.int32, device=gpu_device)
+    offsets = torch.full((65,), -1, dtype=torch.int32, device=gpu_device)
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.moe_a2a_route(None, None, 0, 0, 6, 64, 8, 0, counts.data_ptr(), offsets.data_ptr(), None, None, None,
+                             None, None, 0, st) == 0
+    torch.cuda.synchronize()
+    assert int(counts.abs().sum()) == 0 and int(offsets.abs().sum()) == 0
+    counts.fill_(-1)
+    offsets.fill_(-1)
+    assert lib.moe_a2a_route_dispatch(None, None, None, 0, 0, 6, 64, 8, 2048, 0, counts.data_ptr(),
+                                      offsets.data_ptr(), None, None, None, None, None, st) == 0
+    torch.cuda.synchronize()
+    assert int(counts.abs().sum()) == 0 and int(offsets.abs().sum()) == 0
 
 
 def test_custom_kernel_contract(gpu_device):

@@ -231,3 +231,61 @@ def test_fp8_path_output_within_tolerance_of_bf16_path():
     a = V.run_world(wl.cfg, wl.world, stub_kind=1, fp8=True)["y"].float()
     b = V.run_world(wl.cfg, wl.world, stub_kind=1, fp8=False)["y"].float()
     assert float((a - b).abs().max()) < 2.0 ** -4 * float(b.abs().max())
+
+
+# ---- expert GEMM helpers (no counterpart in the reference: pinned by explicit loops) -----------
+def test_weight_quantisation_and_q8_gemm_against_explicit_loops():
+    """quantize_weights_fp8 / dequantize_weights_fp8 / expert_gemm_q8 on 2 x 128 x 128 integer-valued
+    weights, against plain Python loops over blocks and the independent e4m3fn encoder: the block
+    scale is amax / 448, the bits are the nearest-even e4m3fn code of w / scale, dequantisation is
+    code value x scale, and the product is the sum over K of x x dequantised weight, rounded once."""
+    g = torch.Generator().manual_seed(21)
+    E, N, Kd = 2, 128, 256  # one block row, two K blocks per expert
+    w = torch.randint(-40, 41, (E, N, Kd), generator=g).to(torch.float32)
+    w[1, :, 128:] = 0.0  # an all-zero block: scale 1, codes 0
+    q, s = V.quantize_weights_fp8(w)
+    assert q.dtype == torch.uint8 and tuple(q.shape) == (E, N, Kd) and tuple(s.shape) == (E, 1, 2)
+    tab = e4m3fn_table()
+    deq_loop = np.zeros((E, N, Kd), dtype=np.float64)
+    for e in range(E):
+        for kb in range(2):
+            blk = w[e, :, 128 * kb:128 * (kb + 1)].numpy()
+            amax = np.float32(np.abs(blk).max())
+            scale = np.float32(1.0) if amax == 0 else np.float32(amax / np.float32(448.0))
+            assert np.float32(s[e, 0, kb]) == scale
+            codes = encode_e4m3fn_nearest_even((blk / scale).astype(np.float32))
+            assert np.array_equal(q[e, :, 128 * kb:128 * (kb + 1)].numpy(), codes)
+            deq_loop[e, :, 128 * kb:128 * (kb + 1)] = tab[codes].astype(np.float32) * scale
+    deq = V.dequantize_weights_fp8(q, s)
+    assert np.array_equal(deq.numpy(), deq_loop.astype(np.float32))
+    # integer-valued rows keep every partial sum exact in f32, so the loop below has ONE right answer
+    x = torch.randint(-3, 4, (6, Kd), generator=g).to(torch.bfloat16)
+    offsets = torch.tensor([0, 4, 6], dtype=torch.int32)
+    y = V.expert_gemm_q8(x, None, q, s, offsets, torch.float32)
+    for r in range(6):
+        e = 0 if r < 4 else 1
+        for n in range(0, N, 17):
+            acc = 0.0
+            for k in range(Kd):
+                acc += float(x[r, k]) * float(deq_loop[e, n, k])
+            assert abs(float(y[r, n]) - acc) <= 1e-4 * max(1.0, abs(acc)), (r, n)
+    # fp8 rows: dequantised with their own scales; round_rows rounds them once to the output type first
+    xq, xs = V.quantize_fp8(x)
+    xd = V.dequantize_fp8(xq, xs)
+    for round_rows in (False, True):
+        y8 = V.expert_gemm_q8(xq, xs, q, s, offsets, torch.bfloat16, round_rows=round_rows)
+        rows = xd.to(torch.bfloat16).float() if round_rows else xd
+        for r in (0, 5):
+            e = 0 if r < 4 else 1
+            want = (rows[r].double() @ torch.from_numpy(deq_loop[e]).t()).to(torch.float32).to(torch.bfloat16)
+            assert torch.equal(bits(y8[r]), bits(want)), (round_rows, r)
+
+
+def test_stub_factor_f32_division_equals_the_double_quotient_rounded_to_f32():
+    """The kernels divide (1 + e) by E in f32 (correctly rounded); the oracle divides in double and
+    rounds to f32.  Equal for every expert count the library accepts."""
+    for E in range(1, 1025):
+        e = np.arange(E, dtype=np.int64)
+        via_double = ((1 + e).astype(np.float64) / np.float64(E)).astype(np.float32)
+        via_f32 = (1 + e).astype(np.float32) / np.float32(E)
+        assert np.array_equal(via_double, via_f32), E
