@@ -214,6 +214,7 @@ def summarise(per):
 ROUTE_KERNELS = ("route_tiles", "route_hist", "route_scan", "route_rank")
 DISPATCH_KERNELS = ("dispatch_rows", "route_dispatch", "route_dispatch_tile", "dispatch_fp8")
 COMBINE_KERNELS = ("combine_rows", "stub_combine")
+FORWARD_KERNELS = ("forward_token",)  # dispatch and combine of a token in one launch
 STUB_KERNELS = ("stub_rows", "stub_fp8")
 
 
@@ -307,8 +308,9 @@ class Leg:
 
 def phase_times(per, steps):
     t = dict(route=per_step(per, ROUTE_KERNELS, steps), dispatch=per_step(per, DISPATCH_KERNELS, steps),
-             combine=per_step(per, COMBINE_KERNELS, steps), stub=per_step(per, STUB_KERNELS, steps))
-    t["dc"] = t["route"] + t["dispatch"] + t["combine"]
+             combine=per_step(per, COMBINE_KERNELS, steps), stub=per_step(per, STUB_KERNELS, steps),
+             forward=per_step(per, FORWARD_KERNELS, steps))
+    t["dc"] = t["route"] + t["dispatch"] + t["combine"] + t["forward"]
     return t
 
 
@@ -396,9 +398,12 @@ def main():
     value = b_dc / t["dc"] / 1e3  # bytes/us -> GB/s
 
     # dominant kernel for the roofline entry
-    disp_name = next(n for n in DISPATCH_KERNELS if n in per)
-    comb_name = next(n for n in COMBINE_KERNELS if n in per)
-    cand = [(disp_name, ab["dispatch"]), (comb_name, ab["combine"])]
+    if any(n in per for n in FORWARD_KERNELS):  # one launch moves the bytes of both phases
+        cand = [(next(n for n in FORWARD_KERNELS if n in per), b_dc)]
+    else:
+        disp_name = next(n for n in DISPATCH_KERNELS if n in per)
+        comb_name = next(n for n in COMBINE_KERNELS if n in per)
+        cand = [(disp_name, ab["dispatch"]), (comb_name, ab["combine"])]
     dom_name, dom_bytes = max(cand, key=lambda c: statistics.fmean(per[c[0]]))
     dom_us = statistics.fmean(per[dom_name])
     traffic, traffic_source = measured_traffic(args.workload, dom_name)
@@ -412,7 +417,7 @@ def main():
         ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None, dtype=dtype,
         data="synthetic", config=config,
         dispatch_combine_us=round(t["dc"], 3), route_us=round(t["route"], 3), dispatch_us=round(t["dispatch"], 3),
-        stub_us=round(t["stub"], 3), combine_us=round(t["combine"], 3),
+        stub_us=round(t["stub"], 3), combine_us=round(t["combine"], 3), one_launch_us=round(t["forward"], 3),
         pct_of_hbm_peak=round(100.0 * value / HBM_PEAK_GBPS, 2),
         tokens_per_s=round(T / (t["dc"] * 1e-6), 1),
         tokens_per_s_wall=round(T / (ms_per_step * 1e-3), 1),

@@ -195,7 +195,12 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
  * ref_kernel, all2all/reference.py:256-272).  Same kernels and results as the separate calls;
  * one host call keeps the launches back to back.
  *   fp8_dispatch  0: 16-bit rows, 1: fp8 rows with f32 scales, 2: fp8 rows with power-of-two scales
- *   fuse_stub     0: stub kernel + combine, 1: moe_a2a_stub_combine
+ *   fuse_stub     0: stub kernel + combine, 1: moe_a2a_stub_combine.  With fuse_stub and fuse_route on a
+ *                 small routing table (what moe_a2a_route_dispatch takes one token per workgroup for:
+ *                 a few thousand entries), 16-bit rows of one element type and the compact layout,
+ *                 the whole path is ONE launch: a workgroup dispatches its token and then folds the
+ *                 rows it has just written -- the stand-in expert is elementwise, so a token's result
+ *                 depends on no other workgroup's rows; same buffers, same bits, no launch in between.
  *   fuse_route    0: moe_a2a_route + dispatch, 1: moe_a2a_route_dispatch when moe_a2a_fused_ok,
  *                 2: moe_a2a_route_dispatch at any size
  *   expert_y      [R,H] (padded layout: [E*max_recv,H]) of out_type, unused (may be NULL) when fuse_stub
@@ -207,6 +212,10 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                     int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
                     int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
                     size_t workspace_bytes, moe_a2a_stream_t stream);
+
+/* Kernel launches moe_a2a_forward issues for this shape and these switches (host logic only). */
+int moe_a2a_forward_launches(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch,
+                             int fuse_route, int fuse_stub);
 
 /*
  * Expert compute on the dispatched layout: y[rows of e, :] = x[rows of e, :] * W_e^T for every
@@ -315,7 +324,9 @@ const char* moe_a2a_kernel_name(int kernel_id);
 #define MOE_A2A_OPT_COMBINE_LANES 3 /* lanes of a combine workgroup at cache-resident sizes (64 .. 512)     */
 #define MOE_A2A_OPT_COMBINE_VPL 4   /* 2: two row vectors per lane in the combine at cache-resident sizes   */
 #define MOE_A2A_OPT_TIMER_EVENT_FLAGS 5 /* hipEventCreateWithFlags value for the launch timer's events    */
-#define MOE_A2A_OPT_COUNT 6
+#define MOE_A2A_OPT_COMBINE_PLAIN_MAP 6 /* 1: combine workgroups in token order, not grouped by XCD          */
+#define MOE_A2A_OPT_TWO_LAUNCHES 7      /* 1: moe_a2a_forward never takes its one-launch form                */
+#define MOE_A2A_OPT_COUNT 8
 int moe_a2a_set_option(int option, int value);
 int moe_a2a_get_option(int option);
 

@@ -14,7 +14,8 @@ F16, BF16 = 0, 1
 FP8_SCALE_F32, FP8_SCALE_POW2 = 0, 1
 STATUS_BAD_EXPERT, STATUS_OVERFLOW = 1, 2  # bits of the routing status word
 # option switches of moe_a2a_set_option (0 = the library decides)
-OPT_ROUTE_TILE, OPT_GEMM_TILE, OPT_GEMM_STAGED, OPT_COMBINE_LANES, OPT_COMBINE_VPL, OPT_TIMER_EVENT_FLAGS = range(6)
+(OPT_ROUTE_TILE, OPT_GEMM_TILE, OPT_GEMM_STAGED, OPT_COMBINE_LANES, OPT_COMBINE_VPL, OPT_TIMER_EVENT_FLAGS,
+ OPT_COMBINE_PLAIN_MAP, OPT_TWO_LAUNCHES) = range(8)
 
 _i32p = C.c_void_p  # device pointers travel as plain addresses
 _vp = C.c_void_p
@@ -39,6 +40,7 @@ PROTOTYPES = {
                                     _int, _vp]),
     "moe_a2a_forward": (_int, [_vp, _i32p, _vp, _i32p] + [_int] * 14 + [_i32p] * 6 + [_vp, _vp, _vp, _vp, _vp, C.c_size_t,
                                                                                       _vp]),
+    "moe_a2a_forward_launches": (_int, [_int] * 9),
     "moe_a2a_expert_gemm": (_int, [_vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_expert_gemm_fp8": (_int, [_vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),
     "moe_a2a_expert_gemm_q8": (_int, [_vp, _vp, _vp, _vp, _i32p, _vp, _int, _int, _int, _int, _int, _int, _vp]),

@@ -61,12 +61,13 @@ enum KernelId {
   KID_EXPERT_GEMM_F8,
   KID_EXPERT_GEMM_MX,
   KID_ROUTE_EMPTY,
+  KID_FORWARD_TOKEN,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
-    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty"};
+    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -225,6 +226,12 @@ inline int option(int which) { return g_option[which].load(std::memory_order_rel
 // fewer, wider ones (256 tokens of 896 vectors: 4 x 224 lanes 6.4 us, 2 x 448 lanes 6.7 us); a
 // workgroup keeps at least 128 lanes.  Streaming sizes keep the widest workgroups (512 lanes).
 // MOE_A2A_OPT_COMBINE_LANES / _VPL override both (measurements).
+// The XCD-aware workgroup map of the combine (see combine_body): cache-resident sizes only.
+bool combine_xcd_map(int T, int nsplit, bool streaming) {
+  return !streaming && option(MOE_A2A_OPT_COMBINE_PLAIN_MAP) == 0 &&
+         ((long long)T + kXcds) * nsplit < (long long)INT32_MAX;
+}
+
 CombineGeom combine_geom(int nvec, int T, bool streaming) {
   CombineGeom g;
   g.vpl = 1;
@@ -579,8 +586,9 @@ static int combine_impl(const void* expert_y, const float* weights, const int32_
   const bool st = streams((long long)T * K, T, H, 2, 2);
   const bool through = dispatched_bytes > (256ll << 20);
   const CombineGeom g = combine_geom(nvec, T, st);
-  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
-#define COMBINE_ARGS (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit
+  const int xcd_T = combine_xcd_map(T, g.nsplit, st) ? T : 0;
+  dim3 grid((unsigned)(xcd_T ? ceil_div(T, kXcds) * kXcds : T) * g.nsplit), block(g.threads);
+#define COMBINE_ARGS (const uint4*)expert_y, weights, slot_of_entry, (uint4*)out, K, nvec, g.per, g.nsplit, xcd_T
 #define COMBINE_LAUNCH(EL, MD, KT)                                                                             \
   {                                                                                                            \
     if (st && through)                                                                                         \
@@ -655,9 +663,11 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
   }
   const int nvec = H / 8;
   const CombineGeom g = combine_geom(nvec, T, st);
-  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
-#define SC_ARGS \
-  (const uint4*)disp, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K, nvec, g.per, g.nsplit
+  const int xcd_T = combine_xcd_map(T, g.nsplit, st) ? T : 0;
+  dim3 grid((unsigned)(xcd_T ? ceil_div(T, kXcds) * kXcds : T) * g.nsplit), block(g.threads);
+#define SC_ARGS                                                                                              \
+  (const uint4*)disp, indices, weights, slot_of_entry, (uint4*)out, stub_kind, E, E_l, K, nvec, g.per, g.nsplit, \
+      xcd_T
 #define SC_LAUNCH(IN, OUT, MD, KT)                                                                            \
   {                                                                                                           \
     if (st)                                                                                                   \
@@ -697,6 +707,77 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
 }
 #undef MOE_A2A_SWITCH_KT
 
+// The whole path in one launch (forward_token_kernel): small routing tables, 16-bit rows of one
+// element type, compact layout, stub folded in.
+static bool forward_one_launch_ok(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch) {
+  if (fp8_dispatch || max_recv > 0 || in_type != out_type || !fused_small_ok(T, K, H)) return false;
+  if (option(MOE_A2A_OPT_ROUTE_TILE) == 1 || option(MOE_A2A_OPT_TWO_LAUNCHES) == 1) return false;
+  const RowGeom g = fused_geom(H / 8, T * K);
+  return fused_entries_per_thread(T * K, g.threads) <= 8;
+}
+
+int moe_a2a_forward_launches(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch,
+                             int fuse_route, int fuse_stub) {
+  if (T <= 0) return 0;
+  if (fuse_stub && fuse_route && forward_one_launch_ok(T, K, H, max_recv, in_type, out_type, fp8_dispatch)) return 1;
+  const bool fused = !fp8_dispatch && (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
+  int n = fused ? 1 : 2;  // routing + dispatch
+  if (!fused) {
+    const long long R = (long long)T * K;
+    if (R > kRouteTilesMaxRows) n += ceil_div((int)std::min<long long>(R, INT32_MAX), kRouteThreads) <= kRouteFoldMaxTiles ? 1 : 2;
+  }
+  return n + (fuse_stub ? 1 : 2);
+}
+
+static int forward_one_launch(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
+                              int src_rank, int T, int K, int E, int W, int H, int elem_type, int stub_kind,
+                              int combine_mode, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
+                              int32_t* src_of_slot, int32_t* meta, int32_t* status, void* disp, void* out,
+                              hipStream_t stream) {
+  if (int rc = check_route_shape(T, K, E, W)) return rc;
+  if (int rc = check_rows(x, disp, T, K, H, 8)) return rc;
+  if (!aligned16(out)) return MOE_A2A_E_ALIGN;
+  if (!counts || !offsets || !indices || !weights || !slot_of_entry || !src_of_slot || !meta || !out)
+    return MOE_A2A_E_NULL;
+  RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), 0, counts, offsets,
+              slot_of_entry, src_of_slot, meta, status};
+  const int nvec = H / 8;
+  const RowGeom g = fused_geom(nvec, T * K);
+  const int vpl = fused_vectors_per_lane(nvec);
+  const int ept = fused_entries_per_thread(T * K, g.threads);
+  const int E_l = E / W;
+  dim3 grid((unsigned)T * g.nsplit + 1), block(g.threads);
+#define FWD_ARGS a, (const uint4*)x, (uint4*)disp, weights, (uint4*)out, stub_kind, E_l, nvec, g.per, g.nsplit
+#define FWD4(EPT, VPL, EL, MD)                                                                                   \
+  {                                                                                                              \
+    if (K == 8)                                                                                                  \
+      return launch(KID_FORWARD_TOKEN, forward_token_kernel<EPT, VPL, EL, MD, 8>, grid, block, 0, stream, FWD_ARGS); \
+    return launch(KID_FORWARD_TOKEN, forward_token_kernel<EPT, VPL, EL, MD, 0>, grid, block, 0, stream, FWD_ARGS); \
+  }
+#define FWD3(EPT, VPL, EL)                                                      \
+  {                                                                             \
+    if (combine_mode == MOE_A2A_COMBINE_STRICT) FWD4(EPT, VPL, EL, MOE_A2A_COMBINE_STRICT) \
+    FWD4(EPT, VPL, EL, MOE_A2A_COMBINE_F32)                                     \
+  }
+#define FWD2(EPT, VPL)                          \
+  {                                             \
+    if (elem_type == MOE_A2A_BF16) FWD3(EPT, VPL, Bf16) \
+    FWD3(EPT, VPL, F16)                         \
+  }
+#define FWD1(EPT)             \
+  {                           \
+    if (vpl == 2) FWD2(EPT, 2) \
+    FWD2(EPT, 1)              \
+  }
+  if (ept == 4) FWD1(4)
+  FWD1(8)
+#undef FWD1
+#undef FWD2
+#undef FWD3
+#undef FWD4
+#undef FWD_ARGS
+}
+
 int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
                     int src_rank, int T, int K, int E, int W, int H, int max_recv, int in_type, int out_type,
                     int fp8_dispatch, int stub_kind, int combine_mode, int fuse_route, int fuse_stub,
@@ -707,6 +788,13 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   if (fp8_dispatch < 0 || fp8_dispatch > 2) return MOE_A2A_E_DTYPE;
   if (fp8_dispatch && !disp_scale) return MOE_A2A_E_NULL;
   if (!fuse_stub && T > 0 && !expert_y) return MOE_A2A_E_NULL;
+  if (stub_kind != MOE_A2A_STUB_OWNER_RANK && stub_kind != MOE_A2A_STUB_EXPERT_FRACTION) return MOE_A2A_E_DTYPE;
+  if (combine_mode != MOE_A2A_COMBINE_STRICT && combine_mode != MOE_A2A_COMBINE_F32) return MOE_A2A_E_DTYPE;
+  if (T > 0 && fuse_stub && fuse_route &&
+      forward_one_launch_ok(T, K, H, max_recv, in_type, out_type, fp8_dispatch))
+    return forward_one_launch(x, indices, weights, rank_start, src_rank, T, K, E, W, H, in_type, stub_kind,
+                              combine_mode, counts, offsets, slot_of_entry, src_of_slot, meta, status, disp, out,
+                              (hipStream_t)stream);
   const bool fused = !fp8_dispatch && T > 0 &&
                      (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
   if (fused) {
