@@ -12,7 +12,9 @@ region starts.  Prints ONE JSON line:
                rows; read R rows, write T rows) / summed GPU durations of the routing,
                dispatch and combine kernels of a step.  Kernel durations come from HIP
                events bound to each launch, on the stream the kernels run on.
-  ms_per_step  wall time of a whole step, events around K steps of hipGraph replays.
+  ms_per_step  wall time of a whole step: events around K steps launched back to back from a C loop
+               behind an already filled queue (graph_ms_per_step: the same K steps as hipGraph replays,
+               which pay about 9 us per graph launch on top).
   roofline     the slower of the dispatch / combine kernels against the 8 TB/s HBM peak; `traffic`
                from profiles/traffic.json when that record was taken on the present kernel sources.
   cpu_baseline the CPU oracle (a port of the reference's torch path) timed on the host
@@ -35,6 +37,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+GRAPH_STEPS = 40  # steps captured into one hipGraph
 
 # HBM bytes per launch, measured: profiles/traffic.json holds rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # readings (KiB per dispatch, each scaled by what the same counter reads for a plain 256 MiB device
@@ -91,7 +94,8 @@ def parse_args():
     p.add_argument("--no-fuse-stub", action="store_true",
                    help="expert stub as a launch of its own (the default folds it into the combine, as custom_kernel does)")
     p.add_argument("--graph-only", action="store_true",
-                   help="hipGraph replays of the default configuration and nothing else (the form to run under rocprofv3)")
+                   help="wall-clock legs of the default configuration only (hipGraph replays, then plain launches from "
+                        "the C loop): no launch carries events -- the form to run under rocprofv3")
     p.add_argument("--single", action="store_true", help="skip the legs reported beside the headline (other stub form, f32 combine)")
     p.add_argument("--timer-event-flags", default="", metavar="FLAGS",
                    help="hipEventCreateWithFlags value for the launch timer's events (measurement aid)")
@@ -214,7 +218,7 @@ def summarise(per):
 ROUTE_KERNELS = ("route_tiles", "route_hist", "route_scan", "route_rank")
 DISPATCH_KERNELS = ("dispatch_rows", "route_dispatch", "route_dispatch_tile", "dispatch_fp8")
 COMBINE_KERNELS = ("combine_rows", "stub_combine")
-FORWARD_KERNELS = ("forward_token",)  # dispatch and combine of a token in one launch
+FORWARD_KERNELS = ("forward_token", "forward_tile")  # dispatch and combine of a token in one launch
 STUB_KERNELS = ("stub_rows", "stub_fp8")
 
 
@@ -240,38 +244,78 @@ class Leg:
         self.run_n = None
 
     def graph_wall(self, steps, warmup, use_graph=True):
-        """Wall time per step (ms) of exactly `steps` steps: hipGraph replays (the host class alternates
-        between two buffer sets, so one graph holds two steps; an odd count ends with a one-step graph)."""
+        """Wall time per step (ms) of exactly `steps` steps replayed from hipGraphs of up to
+        GRAPH_STEPS steps each (an even number: the host class alternates between two buffer sets; what
+        is left over ends in a shorter graph).  Inside a graph the launches follow each other with
+        nothing but the GPU's own launch overhead between them, and a graph launch (a few us of
+        host-visible latency) is spread over its steps, so for a configuration whose steps are all
+        dispatch/combine kernels this IS the mean launch-to-launch period of those kernels -- the
+        duration a profiler's kernel trace reports for back-to-back launches."""
         torch, main, step = self.torch, self.main, self.step
-        with torch.cuda.stream(main):
-            run, per_run, tail = step, 1, None
-            if use_graph:
-                per_run = 2
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, stream=main):
-                    step()
+
+        def capture(n):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=main):
+                for _ in range(n):
                     self.y = step()
-                run = graph.replay
-                if steps % 2:
-                    tail = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(tail, stream=main):
-                        self.y = step()
+            return g
+
+        with torch.cuda.stream(main):
+            if use_graph:
+                chunk = min(GRAPH_STEPS, steps - steps % 2) or 1
+                full, rem = capture(chunk), steps % chunk
+                tail = capture(rem) if rem else None
+                n_full = steps // chunk
+                run = full.replay
+            else:
+                chunk, tail, n_full, run = 1, None, steps, step
             # spin-up: the first milliseconds of GPU work after an idle period run below the
             # sustained clocks; 0.3 s of untimed steps come before the W warm-up steps
             t_spin = time.perf_counter()
             while time.perf_counter() - t_spin < 0.3:
-                for _ in range(50):
+                for _ in range(max(1, 100 // chunk)):
                     run()
                 main.synchronize()
-            for _ in range(max(1, warmup // per_run)):
+            for _ in range(max(1, warmup // chunk)):
                 run()
             main.synchronize()
+            # two more untimed replays go out right in front of the timed region: the GPU works on
+            # them while the host enqueues the start event and the timed launches (submitting a graph
+            # of 40 launches takes the host longer than a step takes the GPU), so the K timed steps
+            # start back to back instead of behind an idle queue
+            for _ in range(2):
+                run()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(main)
-            for _ in range(steps // per_run):
+            for _ in range(n_full):
                 run()
             if tail is not None:
                 tail.replay()
+            e1.record(main)
+            main.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    def loop_wall(self, steps, warmup):
+        """Wall time per step (ms) of exactly `steps` steps launched one by one from a C loop (plain
+        launches, no graph): the host issues a launch in a fraction of the time a step takes the GPU,
+        so with a few steps already queued the timed ones run back to back, and there is no graph
+        boundary (about 9 us per hipGraphLaunch here) inside the timed region."""
+        torch, main = self.torch, self.main
+        with torch.cuda.stream(main):
+            if self.run_n is None:
+                self.run_n = c_loop(self.step)
+                self.run_n(4)
+                main.synchronize()
+            t_spin = time.perf_counter()
+            while time.perf_counter() - t_spin < 0.3:  # sustained clocks, as in graph_wall
+                self.run_n(100)
+                main.synchronize()
+            self.run_n(max(1, warmup))
+            main.synchronize()
+            self.run_n(16)  # the queue the timed steps start behind
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(main)
+            self.run_n(steps)
             e1.record(main)
             main.synchronize()
         return e0.elapsed_time(e1) / steps
@@ -306,11 +350,27 @@ class Leg:
         return per, details
 
 
-def phase_times(per, steps):
-    t = dict(route=per_step(per, ROUTE_KERNELS, steps), dispatch=per_step(per, DISPATCH_KERNELS, steps),
-             combine=per_step(per, COMBINE_KERNELS, steps), stub=per_step(per, STUB_KERNELS, steps),
-             forward=per_step(per, FORWARD_KERNELS, steps))
+def phase_times(per, steps, wall_us):
+    """Per-step times of the phases.  `*_kernel` figures are the kernels' own durations (HIP events
+    bound to each launch).  The figures without the suffix add to every launch its share of the
+    launch overhead, (wall clock of a step in the hipGraph - sum of the kernel durations) / launches:
+    the launch-to-launch PERIOD, which is what a profiler's kernel trace reports as the duration of
+    back-to-back launches (it stamps a kernel's start when the one before it ends) and what a caller
+    pays.  `dc` = routing + dispatch + combine; when those are all the launches of a step it equals
+    the wall clock of the step."""
+    names = dict(route=ROUTE_KERNELS, dispatch=DISPATCH_KERNELS, combine=COMBINE_KERNELS, stub=STUB_KERNELS,
+                 forward=FORWARD_KERNELS)
+    t = {}
+    launches = {k: sum(len(per.get(n, [])) for n in v) / steps for k, v in names.items()}
+    kernel = {k: per_step(per, v, steps) for k, v in names.items()}
+    n_all = sum(launches.values())
+    gap = max(0.0, wall_us - sum(kernel.values())) / n_all if n_all else 0.0
+    for k in names:
+        t[k + "_kernel"] = kernel[k]
+        t[k] = kernel[k] + gap * launches[k]
+    t["gap"] = gap
     t["dc"] = t["route"] + t["dispatch"] + t["combine"] + t["forward"]
+    t["dc_kernel"] = kernel["route"] + kernel["dispatch"] + kernel["combine"] + kernel["forward"]
     return t
 
 
@@ -362,27 +422,35 @@ def main():
         str(cfg.in_dtype).replace("torch.", "")]
     config = dict(workload=args.workload, tokens=T, experts=E, top_k=K, hidden=H, emulated_ranks=W, routed_rows=T * K,
                   combine=args.combine,
-                  launch="hipGraph replay, two steps per graph" if use_graph else "eager",
+                  launch="plain launches, back to back from a C loop (ms_per_step); hipGraph replays of up to "
+                         f"{GRAPH_STEPS} steps per graph beside it (graph_ms_per_step)",
                   fused_route=bool(fuse_route and not fp8 and lib.moe_a2a_fused_ok(T, K, H)),
                   fused_stub=bool(fuse_stub),
-                  entry_point="what custom_kernel runs: routing+dispatch, then the combine with the expert stub "
-                              "folded in" if fuse_stub else "routing+dispatch, stub kernel, combine")
+                  launches_per_step=int(lib.moe_a2a_forward_launches(
+                      T, K, H, 0, _lib.BF16, _lib.BF16, 2 if fp8 == "pow2" else int(bool(fp8)), int(fuse_route),
+                      int(fuse_stub))),
+                  entry_point="what custom_kernel runs (moe_a2a_forward with the expert stub folded in)" if fuse_stub
+                  else "routing+dispatch, stub kernel, combine")
 
     # the configuration custom_kernel runs (kernel_amd/submission.py): the expert stand-in folded
     # into the combine, two launches per step at the default workload
     leg = Leg(torch, lib, wl, tensors, main, mode, fp8, fuse_route, fuse_stub)
-    ms_per_step = leg.graph_wall(args.steps, args.warmup, use_graph)
+    graph_ms_per_step = leg.graph_wall(args.steps, args.warmup, use_graph)
+    # the headline wall clock: the same K steps as plain launches from a C loop (no graph boundary in
+    # the timed region; measured 13.67 against 13.96 us per step at K = 20, 13.53 / 13.65 at K = 200)
+    ms_per_step = leg.loop_wall(args.steps, args.warmup)
 
     if args.graph_only:
-        # Nothing but the graph replays above: no event-carrying launch, no second configuration.  This
-        # is the form to put under `rocprofv3 --kernel-trace --stats`, whose per-kernel averages then
-        # describe exactly these launches.  `value` is the wall-clock figure, which includes the idle
-        # time between launches: a lower bound of the kernels' own rate.
+        # Nothing but the two wall-clock measurements above: no event-carrying launch, no second
+        # configuration.  This is the form to put under `rocprofv3 --kernel-trace --stats`, whose
+        # per-kernel averages then describe exactly these launches.  `value` is the wall-clock figure,
+        # which includes the launch overhead between kernels: a lower bound of the kernels' own rate.
         wall_us = ms_per_step * 1e3
         out = dict(metric=METRIC, value=round(b_dc / wall_us / 1e3, 1), unit="GB/s", n_gpus=1, steps=args.steps,
-                   warmup=args.warmup, ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak",
-                   vs_baseline=None, dtype=dtype, data="synthetic",
-                   config=dict(config, launch="hipGraph replay only; value from the wall clock of whole steps"),
+                   warmup=args.warmup, ms_per_step=round(ms_per_step, 6), graph_ms_per_step=round(graph_ms_per_step, 6),
+                   higher_is_better=True, scaling="weak", vs_baseline=None, dtype=dtype, data="synthetic",
+                   config=dict(config, launch="hipGraph replays, then the same steps as plain launches from a C loop; "
+                                              "no launch carries events; value from the wall clock of whole steps"),
                    bytes=dict(dispatch=ab["dispatch"], combine=ab["combine"], stub=ab["stub"]),
                    roofline=None, cpu_baseline=None)
         if args.calibrate_copy:
@@ -394,7 +462,8 @@ def main():
     if args.dump_times:
         with open(args.dump_times, "w") as f:
             json.dump({**per, "_wall_us_per_step_of_the_timed_passes": [det["wall_us_per_step"]]}, f)
-    t = phase_times(per, args.steps)
+    wall_us = ms_per_step * 1e3
+    t = phase_times(per, args.steps, wall_us)
     value = b_dc / t["dc"] / 1e3  # bytes/us -> GB/s
 
     # dominant kernel for the roofline entry
@@ -405,12 +474,16 @@ def main():
         comb_name = next(n for n in COMBINE_KERNELS if n in per)
         cand = [(disp_name, ab["dispatch"]), (comb_name, ab["combine"])]
     dom_name, dom_bytes = max(cand, key=lambda c: statistics.fmean(per[c[0]]))
-    dom_us = statistics.fmean(per[dom_name])
+    dom_kernel_us = statistics.fmean(per[dom_name])
+    dom_us = dom_kernel_us + t["gap"]
     traffic, traffic_source = measured_traffic(args.workload, dom_name)
     roofline = dict(bound="hbm", kernel=dom_name, achieved=round(dom_bytes / dom_us / 1e3, 1), peak=HBM_PEAK_GBPS,
                     unit="GB/s", frac=round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
-                    bytes_per_launch=dom_bytes, avg_us=round(dom_us, 3), traffic=traffic,
-                    traffic_source=traffic_source)
+                    bytes_per_launch=dom_bytes, avg_us=round(dom_us, 3),
+                    avg_us_is="launch-to-launch period in the hipGraph: the kernel's own duration from its HIP "
+                              "events plus its share of the launch overhead (what a profiler's kernel trace "
+                              "reports for back-to-back launches)",
+                    kernel_only_us=round(dom_kernel_us, 3), traffic=traffic, traffic_source=traffic_source)
 
     out = dict(
         metric=METRIC, value=round(value, 1), unit="GB/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
@@ -418,10 +491,14 @@ def main():
         data="synthetic", config=config,
         dispatch_combine_us=round(t["dc"], 3), route_us=round(t["route"], 3), dispatch_us=round(t["dispatch"], 3),
         stub_us=round(t["stub"], 3), combine_us=round(t["combine"], 3), one_launch_us=round(t["forward"], 3),
+        launch_overhead_us_per_launch=round(t["gap"], 3),
         pct_of_hbm_peak=round(100.0 * value / HBM_PEAK_GBPS, 2),
+        kernel_only=dict(dispatch_combine_us=round(t["dc_kernel"], 3),
+                         pct_of_hbm_peak=round(100.0 * b_dc / t["dc_kernel"] / 1e3 / HBM_PEAK_GBPS, 2),
+                         what="sum of the kernels' own durations (HIP events), launch overhead left out"),
         tokens_per_s=round(T / (t["dc"] * 1e-6), 1),
         tokens_per_s_wall=round(T / (ms_per_step * 1e-3), 1),
-        eager_ms_per_step=round(det["eager_ms_per_step"], 6),
+        graph_ms_per_step=round(graph_ms_per_step, 6),
         timed_passes={k: v for k, v in det.items() if k != "eager_ms_per_step"},
         bytes=dict(dispatch=ab["dispatch"], combine=ab["combine"], stub=ab["stub"]),
         kernels=summarise(per),
@@ -431,26 +508,30 @@ def main():
     if not args.single:
         # The same path with the expert stand-in as a launch of its own (three launches per step; the
         # stub's time is then outside dispatch+combine) ...
-        other = Leg(torch, lib, wl, tensors, main, mode, fp8, fuse_route, not fuse_stub)
-        o_ms = other.graph_wall(args.steps, args.warmup, use_graph)
-        o_per, _ = other.kernels(args.steps, args.warmup, o_ms * 1e3)
-        ot = phase_times(o_per, args.steps)
-        out["stub_folded_into_combine" if not fuse_stub else "stub_as_its_own_launch"] = dict(
-            dispatch_combine_us=round(ot["dc"], 3), dispatch_us=round(ot["dispatch"] + ot["route"], 3),
-            stub_us=round(ot["stub"], 3), combine_us=round(ot["combine"], 3), ms_per_step=round(o_ms, 6),
-            value=round(b_dc / ot["dc"] / 1e3, 1), pct_of_hbm_peak=round(100.0 * b_dc / ot["dc"] / 1e3 / HBM_PEAK_GBPS, 2))
-        del other
+        # Beside the headline: the same path with the expert stand-in as a launch of its own; when the
+        # headline ran in one launch, its two-launch form (routing+dispatch, then the combine with the
+        # stub folded in); and the f32-accumulating combine (one rounding at the end: within the
+        # rtol = atol = 1e-2 bar instead of bit-identical to the reference's per-step rounding).
+        legs = [("stub_as_its_own_launch" if fuse_stub else "stub_folded_into_combine", mode, not fuse_stub)]
+        if fuse_stub and t["forward"] > 0:
+            legs.insert(0, ("two_launches", mode, True))
         if mode == contract.COMBINE_STRICT:
-            # ... and with the f32-accumulating combine (one rounding at the end; within the
-            # rtol = atol = 1e-2 bar instead of bit-identical to the reference's per-step rounding):
-            # reported beside the headline value, never in place of it.
-            l32 = Leg(torch, lib, wl, tensors, main, contract.COMBINE_F32, fp8, fuse_route, fuse_stub)
-            p32, _ = l32.kernels(args.steps, args.warmup, ms_per_step * 1e3)
-            t32 = phase_times(p32, args.steps)
-            out["f32_combine"] = dict(dispatch_combine_us=round(t32["dc"], 3), combine_us=round(t32["combine"], 3),
-                                      value=round(b_dc / t32["dc"] / 1e3, 1),
-                                      pct_of_hbm_peak=round(100.0 * b_dc / t32["dc"] / 1e3 / HBM_PEAK_GBPS, 2))
-            del l32
+            legs.append(("f32_combine", contract.COMBINE_F32, fuse_stub))
+        for name, leg_mode, leg_fuse in legs:
+            lib.moe_a2a_set_option(_lib.OPT_TWO_LAUNCHES, 0 if name == "f32_combine" else 1)
+            other = Leg(torch, lib, wl, tensors, main, leg_mode, fp8, fuse_route, leg_fuse)
+            o_ms = other.loop_wall(args.steps, args.warmup)
+            o_per, _ = other.kernels(args.steps, args.warmup, o_ms * 1e3)
+            ot = phase_times(o_per, args.steps, o_ms * 1e3)
+            out[name] = dict(
+                dispatch_combine_us=round(ot["dc"], 3), dispatch_us=round(ot["dispatch"] + ot["route"], 3),
+                stub_us=round(ot["stub"], 3), combine_us=round(ot["combine"], 3),
+                one_launch_us=round(ot["forward"], 3), ms_per_step=round(o_ms, 6),
+                value=round(b_dc / ot["dc"] / 1e3, 1),
+                pct_of_hbm_peak=round(100.0 * b_dc / ot["dc"] / 1e3 / HBM_PEAK_GBPS, 2),
+                kernel_only_dispatch_combine_us=round(ot["dc_kernel"], 3))
+            del other
+        lib.moe_a2a_set_option(_lib.OPT_TWO_LAUNCHES, 0)
 
     if args.cold:
         # cold caches: overwrite 1 GiB (4x the 256 MB Infinity Cache) before every step
@@ -460,7 +541,7 @@ def main():
             flush.fill_(1)
             leg.run_n(2)
             perc = kernel_times(lib, leg.run_n, n_cold, torch, before_each=lambda: flush.fill_(1))
-        tc = per_step(perc, ROUTE_KERNELS + DISPATCH_KERNELS + COMBINE_KERNELS, n_cold)
+        tc = per_step(perc, ROUTE_KERNELS + DISPATCH_KERNELS + COMBINE_KERNELS + FORWARD_KERNELS, n_cold)
         out["cold"] = dict(dispatch_combine_us=round(tc, 3), GBps=round(b_dc / tc / 1e3, 1),
                            pct_of_hbm_peak=round(100.0 * b_dc / tc / 1e3 / HBM_PEAK_GBPS, 2),
                            kernels={k: v["mean_us"] for k, v in summarise(perc).items()})
@@ -485,6 +566,7 @@ def calibrate_copy(torch, main, dev):
 
 
 KERNEL_OF_SYMBOL = (("route_dispatch_tile_kernel", "route_dispatch_tile"), ("route_dispatch_kernel", "route_dispatch"),
+                    ("forward_token_kernel", "forward_token"), ("forward_tile_kernel", "forward_tile"),
                     ("stub_combine_rows_kernel", "stub_combine"), ("stub_combine_fp8_kernel", "stub_combine"),
                     ("combine_rows_kernel", "combine_rows"), ("dispatch_rows_kernel", "dispatch_rows"),
                     ("dispatch_fp8_kernel", "dispatch_fp8"), ("stub_rows_kernel", "stub_rows"),

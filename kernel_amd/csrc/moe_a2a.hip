@@ -29,6 +29,7 @@
 namespace {
 
 constexpr int kWave = 64;
+constexpr int kXcds = 8;  // accelerator dies of an MI355X; workgroup b runs on die b % 8
 constexpr int kRouteThreads = 1024;
 constexpr int kRouteWaves = kRouteThreads / kWave;
 constexpr int kRouteTilesMaxRows = 32 * kRouteThreads;  // one-launch routing up to here (8.7 against 10.2 us in two
@@ -62,12 +63,13 @@ enum KernelId {
   KID_EXPERT_GEMM_MX,
   KID_ROUTE_EMPTY,
   KID_FORWARD_TOKEN,
+  KID_FORWARD_TILE,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
-    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token"};
+    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token", "forward_tile"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -709,11 +711,19 @@ int moe_a2a_stub_combine(const void* disp, const float* disp_scale, const int32_
 
 // The whole path in one launch (forward_token_kernel): small routing tables, 16-bit rows of one
 // element type, compact layout, stub folded in.
+// 0: no; 1: one token per workgroup (forward_token_kernel); 2: a tile of tokens per workgroup
+// (forward_tile_kernel), wherever moe_a2a_route_dispatch would take its token-tile kernel by itself.
+static int forward_one_launch_form(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch) {
+  if (fp8_dispatch || max_recv > 0 || in_type != out_type || T < 1) return 0;
+  if (option(MOE_A2A_OPT_TWO_LAUNCHES) == 1 || !moe_a2a_fused_ok(T, K, H)) return 0;
+  if (fused_small_ok(T, K, H) && option(MOE_A2A_OPT_ROUTE_TILE) != 1) {
+    const RowGeom g = fused_geom(H / 8, T * K);
+    if (fused_entries_per_thread(T * K, g.threads) <= 8) return 1;
+  }
+  return K <= kTileMaxOwn ? 2 : 0;
+}
 static bool forward_one_launch_ok(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch) {
-  if (fp8_dispatch || max_recv > 0 || in_type != out_type || !fused_small_ok(T, K, H)) return false;
-  if (option(MOE_A2A_OPT_ROUTE_TILE) == 1 || option(MOE_A2A_OPT_TWO_LAUNCHES) == 1) return false;
-  const RowGeom g = fused_geom(H / 8, T * K);
-  return fused_entries_per_thread(T * K, g.threads) <= 8;
+  return forward_one_launch_form(T, K, H, max_recv, in_type, out_type, fp8_dispatch) != 0;
 }
 
 int moe_a2a_forward_launches(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch,
@@ -742,10 +752,34 @@ static int forward_one_launch(const void* x, const int32_t* indices, const float
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), 0, counts, offsets,
               slot_of_entry, src_of_slot, meta, status};
   const int nvec = H / 8;
+  const int E_l = E / W;
+  if (forward_one_launch_form(T, K, H, 0, elem_type, elem_type, 0) == 2) {
+    const int tile = tile_tokens(T, K, H);
+    dim3 grid((unsigned)ceil_div(T, tile)), block(kTileThreads);
+#define FWT_ARGS a, (const uint4*)x, (uint4*)disp, weights, (uint4*)out, stub_kind, E_l, nvec, tile
+#define FWT3(EL, MD)                                                                                              \
+  {                                                                                                               \
+    switch (K) {                                                                                                  \
+      case 4: return launch(KID_FORWARD_TILE, forward_tile_kernel<EL, MD, 4>, grid, block, 0, stream, FWT_ARGS);  \
+      case 6: return launch(KID_FORWARD_TILE, forward_tile_kernel<EL, MD, 6>, grid, block, 0, stream, FWT_ARGS);  \
+      case 8: return launch(KID_FORWARD_TILE, forward_tile_kernel<EL, MD, 8>, grid, block, 0, stream, FWT_ARGS);  \
+      default: return launch(KID_FORWARD_TILE, forward_tile_kernel<EL, MD, 0>, grid, block, 0, stream, FWT_ARGS); \
+    }                                                                                                             \
+  }
+#define FWT2(EL)                                                        \
+  {                                                                     \
+    if (combine_mode == MOE_A2A_COMBINE_STRICT) FWT3(EL, MOE_A2A_COMBINE_STRICT) \
+    FWT3(EL, MOE_A2A_COMBINE_F32)                                       \
+  }
+    if (elem_type == MOE_A2A_BF16) FWT2(Bf16)
+    FWT2(F16)
+#undef FWT2
+#undef FWT3
+#undef FWT_ARGS
+  }
   const RowGeom g = fused_geom(nvec, T * K);
   const int vpl = fused_vectors_per_lane(nvec);
   const int ept = fused_entries_per_thread(T * K, g.threads);
-  const int E_l = E / W;
   dim3 grid((unsigned)T * g.nsplit + 1), block(g.threads);
 #define FWD_ARGS a, (const uint4*)x, (uint4*)disp, weights, (uint4*)out, stub_kind, E_l, nvec, g.per, g.nsplit
 #define FWD4(EPT, VPL, EL, MD)                                                                                   \

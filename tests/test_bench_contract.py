@@ -47,9 +47,43 @@ def test_json_line_has_the_contract_keys(gpu_device):
     assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
     assert r["traffic"] is None or r["traffic"] > 0
-    # the kernel-time figure cannot beat the memory system, and a step's wall time holds its kernels
+    assert isinstance(r["traffic_source"], str) and r["traffic_source"]
+    # the headline times what custom_kernel runs, and says how many launches that is
+    assert d["config"]["fused_stub"] is True and d["config"]["launches_per_step"] >= 1
+    # the figure cannot beat the memory system; a step's wall time holds its kernels and their launch
+    # overhead, so the period-based figure cannot beat the kernels' own durations either
     assert 0 < d["value"] < 8000.0
-    assert d["ms_per_step"] * 1e3 >= d["dispatch_combine_us"]
+    assert d["ms_per_step"] * 1e3 >= d["dispatch_combine_us"] - 0.01
+    assert d["dispatch_combine_us"] >= d["kernel_only"]["dispatch_combine_us"] - 0.01
+    assert abs(r["avg_us"] - (r["kernel_only_us"] + d["launch_overhead_us_per_launch"])) < 0.01
     c = d["cpu_baseline"]
     assert c["kind"] in ("port", "reference") and c["cores"] >= 1 and c["value"] > 0 and c["sample"]
     assert c["gpu_output_bit_identical"] is True
+
+
+def test_traffic_record_counts_only_for_the_sources_it_was_measured_on(tmp_path):
+    """roofline.traffic comes from profiles/traffic.json and is null, with the reason, unless the
+    record names this workload and kernel and was taken on the present kernel sources."""
+    sys.path.insert(0, ROOT)
+    import bench
+
+    now = bench.kernel_source_hash()
+    rec = dict(factor=dict(FETCH_SIZE=2.0, WRITE_SIZE=1.0),
+               entries=[dict(workload="dsv3_rank", kernel="forward_token", symbol="forward_token_kernel<...>",
+                             fetch_kib=100.0, write_kib=200.0, bytes=409600, source_hash=now, commit="abc"),
+                        dict(workload="skew_world", kernel="combine_rows", fetch_kib=1.0, write_kib=1.0, bytes=3072,
+                             source_hash="0000000000000000", commit="abc")])
+    path = tmp_path / "traffic.json"
+    path.write_text(json.dumps(rec))
+    got, why = bench.measured_traffic("dsv3_rank", "forward_token", str(path))
+    assert got == 409600 and "profiles/traffic.json" in why and now in why
+    got, why = bench.measured_traffic("skew_world", "combine_rows", str(path))
+    assert got is None and "other kernel sources" in why  # stale: measured on different code
+    got, why = bench.measured_traffic("dsv3_rank", "route_dispatch", str(path))
+    assert got is None and "no record" in why
+    got, why = bench.measured_traffic("dsv3_rank", "forward_token", str(tmp_path / "missing.json"))
+    assert got is None and "missing" in why
+    # the committed record, if there is one, parses and names its sources
+    if os.path.exists(bench.TRAFFIC_FILE):
+        for e in json.load(open(bench.TRAFFIC_FILE))["entries"]:
+            assert {"workload", "kernel", "bytes", "source_hash", "commit", "fetch_kib", "write_kib"} <= set(e)

@@ -330,6 +330,62 @@ def test_forward_single_call_equals_separate_calls(gpu_device, name):
                 assert_same("slot_of_entry (planned)", ata.last.slot_of_entry, want["slot_of_entry"])
 
 
+@pytest.mark.parametrize("W,E,K,H,tokens", [
+    (1, 8, 2, 256, [64]),                        # tiny: K without a specialised fold
+    (8, 256, 8, 7168, [256, 0, 0, 0, 0, 0, 0, 0]),  # headline shape: one token per workgroup
+    (2, 16, 3, 2880, [100, 37]),                 # rows of 360 vectors (not whole waves), odd K
+    (8, 64, 6, 2048, [128] * 8),                 # a tile of tokens per workgroup
+    (4, 32, 4, 4096, [700, 0, 123, 9]),          # ragged ranks, tiles
+    (1, 4, 1, 64, [5]),                          # K = 1
+    (2, 64, 32, 512, [40, 41]),                  # K = 32: every lane group of the fold is used
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("mode", [C.COMBINE_STRICT, C.COMBINE_F32], ids=["strict", "f32"])
+def test_one_launch_forward_equals_the_oracle_and_the_two_launch_form(gpu_device, options, W, E, K, H, tokens,
+                                                                      dtype, mode):
+    """forward with the stub folded in runs in ONE launch for these shapes (a workgroup dispatches
+    its tokens and then folds the rows it wrote): the dispatched buffers and the output are bit for
+    bit those of the oracle and of the two-launch form of the same call."""
+    g = torch.Generator().manual_seed(sum(tokens) + E + K)
+    cfg = C.MoEConfig(E, K, H, max(tokens) + 1, dtype, dtype)
+    world = []
+    for n in tokens:
+        idx = (torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(n)]).to(torch.int32) if n
+               else torch.empty(0, K, dtype=torch.int32))
+        world.append(C.RankData(n, idx, torch.rand(n, K, generator=g), torch.randn(n, H, generator=g).to(dtype)))
+    x, idx, w, rs = concat_world(world, gpu_device)
+    T = x.shape[0]
+    lib = _lib.load()
+    assert lib.moe_a2a_forward_launches(T, K, H, 0, _lib.BF16, _lib.BF16, 0, 1, 1) == 1
+    for stub_kind in (C.STUB_OWNER_RANK, C.STUB_EXPERT_FRACTION):
+        want = V.run_world(cfg, world, stub_kind=stub_kind, combine_mode=mode)
+        got = {}
+        for two in (0, 1):
+            options.set("TWO_LAUNCHES", two)
+            ata = HipAllToAll(cfg, 0, W, stub_kind=stub_kind, combine_mode=mode, fuse_stub=True)
+            for _ in range(2):
+                y = ata.forward(x, idx, w, rs)
+            torch.cuda.synchronize()
+            d = ata.last
+            assert int(d.status.item()) == 0
+            for key, val in (("counts", d.counts), ("offsets", d.offsets), ("slot_of_entry", d.slot_of_entry),
+                             ("src_of_slot", d.src_of_slot), ("meta", d.meta), ("disp_x", d.disp_x), ("y", y)):
+                assert_same(f"{key} ({'two launches' if two else 'one launch'})", val, want[key])
+            got[two] = y.clone()
+        assert torch.equal(bits(got[0]), bits(got[1]))
+    # the launch timer names the kernel that ran
+    options.set("TWO_LAUNCHES", 0)
+    ata = HipAllToAll(cfg, 0, W, combine_mode=mode, fuse_stub=True)
+    ata.forward(x, idx, w, rs)
+    torch.cuda.synchronize()
+    import ctypes
+    assert lib.moe_a2a_timer_begin(4) == 0
+    ata.forward(x, idx, w, rs)
+    ids, us = (ctypes.c_int * 4)(), (ctypes.c_float * 4)()
+    assert lib.moe_a2a_timer_end(ids, us, 4) == 1
+    assert lib.moe_a2a_kernel_name(ids[0]) in (b"forward_token", b"forward_tile")
+
+
 @pytest.mark.parametrize("name", GOLDEN_CASES)
 @pytest.mark.parametrize("fuse_route", ["always", False])
 def test_padded_layout_is_the_reference_dispatch_return_value(gpu_device, name, fuse_route):
