@@ -67,6 +67,7 @@ extern "C" {
 #define MOE_A2A_E_WORKSPACE (-4) /* workspace missing or smaller than workspace_bytes */
 #define MOE_A2A_E_ALIGN (-5)     /* a row buffer is not 16-byte aligned               */
 #define MOE_A2A_E_STATE (-6)     /* launch timer used out of order                    */
+#define MOE_A2A_E_CAPACITY (-7)  /* table beyond the static scratch of moe_a2a_route_noalloc */
 
 typedef void* moe_a2a_stream_t; /* hipStream_t */
 
@@ -120,6 +121,26 @@ int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_ran
  */
 int moe_a2a_dispatch(const void* x, const int32_t* slot_of_entry, void* disp_x, int T, int K, int H,
                      moe_a2a_stream_t stream);
+
+/*
+ * moe_a2a_route for callers that cannot allocate and have no workspace to hand in: code under hipGraph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose torch code allocates in every call).  Same arguments, kernels and results as
+ * moe_a2a_route, minus the workspace: the (tile, expert) count matrix that routing of more than 32 768
+ * entries needs lives in a static device array of the library instead (4 MiB per GPU, held until the
+ * process ends; smaller tables need no scratch at all).  The call allocates and frees nothing.
+ *   limit   ceil(T*K / 1024) * E <= moe_a2a_route_noalloc_max_ints() (2^20), else MOE_A2A_E_CAPACITY
+ *           and nothing is launched
+ *   sharing every call on a GPU uses that GPU's one array: calls that overlap in time on one GPU (two
+ *           streams, two threads) race on it; calls on one stream do not.  Nothing has to be cleared
+ *           between calls: every cell a call reads, the same call has written.
+ *   set-up  the array's address is looked up on the first call on each device (no stream work, no
+ *           allocation); make that first call outside graph capture.
+ */
+int moe_a2a_route_noalloc(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
+                          int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
+                          int32_t* src_of_slot, int32_t* meta, int32_t* status, moe_a2a_stream_t stream);
+size_t moe_a2a_route_noalloc_max_ints(void);
 
 /*
  * Name of the kernel moe_a2a_route launches first for T tokens of top-K ("route_empty",

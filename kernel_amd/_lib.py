@@ -28,6 +28,9 @@ PROTOTYPES = {
     "moe_a2a_workspace_bytes": (C.c_size_t, [_int, _int, _int]),
     "moe_a2a_route": (_int, [_i32p, _i32p, _int, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p, _i32p, _i32p,
                              _i32p, _vp, C.c_size_t, _vp]),
+    "moe_a2a_route_noalloc": (_int, [_i32p, _i32p, _int, _int, _int, _int, _int, _int, _i32p, _i32p, _i32p, _i32p,
+                                     _i32p, _i32p, _vp]),
+    "moe_a2a_route_noalloc_max_ints": (C.c_size_t, []),
     "moe_a2a_dispatch": (_int, [_vp, _i32p, _vp, _int, _int, _int, _vp]),
     "moe_a2a_fused_max_rows": (_int, []),
     "moe_a2a_fused_ok": (_int, [_int, _int, _int]),

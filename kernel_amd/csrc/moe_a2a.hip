@@ -26,6 +26,12 @@
 
 #include "moe_a2a.h"
 
+// Scratch of moe_a2a_route_noalloc: the (tile, expert) count matrix of the multi-launch routing, held
+// by every GPU the library runs on from load to the end of the process (4 MiB).  In host code this
+// name is only a handle for hipGetSymbolAddress; kernels get the device address it resolves to.
+constexpr size_t kStaticScratchInts = (size_t)1 << 20;
+static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+
 namespace {
 
 constexpr int kWave = 64;
@@ -294,6 +300,9 @@ const char* moe_a2a_strerror(int code) {
     case MOE_A2A_E_WORKSPACE: return "moe_a2a: workspace missing or too small";
     case MOE_A2A_E_ALIGN: return "moe_a2a: row buffer not 16-byte aligned";
     case MOE_A2A_E_STATE: return "moe_a2a: launch timer used out of order";
+    case MOE_A2A_E_CAPACITY:
+      return "moe_a2a: routing table too large for the static scratch of moe_a2a_route_noalloc "
+             "(ceil(T*K/1024) * E must not exceed moe_a2a_route_noalloc_max_ints())";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -315,10 +324,30 @@ static int route_first_kernel(int T, int K) {
   return R <= kRouteTilesMaxRows ? KID_ROUTE_TILES : KID_ROUTE_HIST;
 }
 
-int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
-                  int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
-                  int32_t* meta, int32_t* status, void* workspace, size_t workspace_bytes,
-                  moe_a2a_stream_t stream_) {
+// Device address of `scratch` on the current device, resolved once per device (each GPU holds its
+// own copy of the array at its own address).
+static int static_scratch(int32_t** out) {
+  static std::atomic<int32_t*> resolved[kMaxDevices];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return MOE_A2A_E_STATE;
+  int32_t* p = resolved[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* addr = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)); e != hipSuccess) return (int)e;
+    if (!addr) return MOE_A2A_E_STATE;
+    p = static_cast<int32_t*>(addr);
+    resolved[dev].store(p, std::memory_order_release);  // racing first calls resolve the same address
+  }
+  *out = p;
+  return 0;
+}
+
+// workspace == nullptr and static_ok: the count matrix of a large table goes to the static scratch
+static int route_impl(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
+                      int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
+                      int32_t* meta, int32_t* status, void* workspace, size_t workspace_bytes, bool static_ok,
+                      moe_a2a_stream_t stream_) {
   if (int rc = check_route_shape(T, K, E, W)) return rc;
   if (max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
   if (!counts || !offsets) return MOE_A2A_E_NULL;
@@ -338,9 +367,33 @@ int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_ran
     return launch(KID_ROUTE_TILES, route_tiles_kernel, dim3(ceil_div(a.R, kRouteThreads)), dim3(kRouteThreads), lds,
                   stream, a);
   }
+  if (static_ok) {
+    const size_t need = (size_t)ceil_div(a.R, kRouteThreads) * (size_t)E;
+    if (need > kStaticScratchInts) return MOE_A2A_E_CAPACITY;
+    int32_t* tile = nullptr;
+    if (int rc = static_scratch(&tile)) return rc;
+    return route_large(a, tile, stream);
+  }
   if (!workspace || workspace_bytes < moe_a2a_workspace_bytes(T, K, E)) return MOE_A2A_E_WORKSPACE;
   return route_large(a, (int32_t*)workspace, stream);
 }
+
+int moe_a2a_route(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
+                  int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
+                  int32_t* meta, int32_t* status, void* workspace, size_t workspace_bytes,
+                  moe_a2a_stream_t stream) {
+  return route_impl(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry, src_of_slot,
+                    meta, status, workspace, workspace_bytes, false, stream);
+}
+
+int moe_a2a_route_noalloc(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
+                          int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
+                          int32_t* src_of_slot, int32_t* meta, int32_t* status, moe_a2a_stream_t stream) {
+  return route_impl(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry, src_of_slot,
+                    meta, status, nullptr, 0, true, stream);
+}
+
+size_t moe_a2a_route_noalloc_max_ints(void) { return kStaticScratchInts; }
 
 static int check_rows(const void* a, const void* b, int T, int K, int H, int mult) {
   if (T < 0 || K < 1 || K > MOE_A2A_MAX_TOPK || H < mult || H % mult != 0) return MOE_A2A_E_SHAPE;
