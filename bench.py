@@ -218,7 +218,7 @@ def summarise(per):
 ROUTE_KERNELS = ("route_tiles", "route_hist", "route_scan", "route_rank")
 DISPATCH_KERNELS = ("dispatch_rows", "route_dispatch", "route_dispatch_tile", "dispatch_fp8")
 COMBINE_KERNELS = ("combine_rows", "stub_combine")
-FORWARD_KERNELS = ("forward_token", "forward_tile")  # dispatch and combine of a token in one launch
+FORWARD_KERNELS = ("forward_token", "forward_tile", "dispatch_fold")  # dispatch and combine of a token in one launch
 STUB_KERNELS = ("stub_rows", "stub_fp8")
 
 
@@ -415,7 +415,9 @@ def main():
     # stream carry implicit waits on every other stream of the process.
     main = torch.cuda.Stream()
     main.wait_stream(torch.cuda.current_stream())
-    ab = contract.algorithmic_bytes(T, K, H, 2, 2, fp8)
+    # with the stub folded in, the combine reads the dispatched rows themselves (fp8 bytes and scales
+    # after an fp8 dispatch, not 16-bit expert rows)
+    ab = contract.algorithmic_bytes(T, K, H, 2, 2, fp8, stub_folded=fuse_stub)
     b_dc = ab["dispatch"] + ab["combine"]
     use_graph = not args.no_graph
     dtype = "fp8-e4m3 dispatch, bf16 combine" if fp8 else {"bfloat16": "bf16", "float16": "f16"}[
@@ -523,12 +525,14 @@ def main():
             o_ms = other.loop_wall(args.steps, args.warmup)
             o_per, _ = other.kernels(args.steps, args.warmup, o_ms * 1e3)
             ot = phase_times(o_per, args.steps, o_ms * 1e3)
+            o_ab = contract.algorithmic_bytes(T, K, H, 2, 2, fp8, stub_folded=leg_fuse)
+            o_bytes = o_ab["dispatch"] + o_ab["combine"]
             out[name] = dict(
                 dispatch_combine_us=round(ot["dc"], 3), dispatch_us=round(ot["dispatch"] + ot["route"], 3),
                 stub_us=round(ot["stub"], 3), combine_us=round(ot["combine"], 3),
                 one_launch_us=round(ot["forward"], 3), ms_per_step=round(o_ms, 6),
-                value=round(b_dc / ot["dc"] / 1e3, 1),
-                pct_of_hbm_peak=round(100.0 * b_dc / ot["dc"] / 1e3 / HBM_PEAK_GBPS, 2),
+                bytes=o_bytes, value=round(o_bytes / ot["dc"] / 1e3, 1),
+                pct_of_hbm_peak=round(100.0 * o_bytes / ot["dc"] / 1e3 / HBM_PEAK_GBPS, 2),
                 kernel_only_dispatch_combine_us=round(ot["dc_kernel"], 3))
             del other
         lib.moe_a2a_set_option(_lib.OPT_TWO_LAUNCHES, 0)
@@ -567,6 +571,7 @@ def calibrate_copy(torch, main, dev):
 
 KERNEL_OF_SYMBOL = (("route_dispatch_tile_kernel", "route_dispatch_tile"), ("route_dispatch_kernel", "route_dispatch"),
                     ("forward_token_kernel", "forward_token"), ("forward_tile_kernel", "forward_tile"),
+                    ("dispatch_fold_kernel", "dispatch_fold"),
                     ("stub_combine_rows_kernel", "stub_combine"), ("stub_combine_fp8_kernel", "stub_combine"),
                     ("combine_rows_kernel", "combine_rows"), ("dispatch_rows_kernel", "dispatch_rows"),
                     ("dispatch_fp8_kernel", "dispatch_fp8"), ("stub_rows_kernel", "stub_rows"),
@@ -618,7 +623,8 @@ def record_traffic(directory):
             if name is None:
                 continue
             f_kib, w_kib = statistics.median(fetch[symbol]), statistics.median(write[symbol])
-            entries.append(dict(workload=workload, kernel=name, symbol=symbol.split("(")[0][:120],
+            entries.append(dict(workload=workload, kernel=name,
+                                symbol=symbol.replace("void ", "").replace("(anonymous namespace)::", "")[:100],
                                 fetch_kib=round(f_kib, 1), write_kib=round(w_kib, 1),
                                 bytes=int((f_kib * factor["FETCH_SIZE"] + w_kib * factor["WRITE_SIZE"]) * 1024),
                                 launches=len(fetch[symbol]), source_hash=src, commit=commit))

@@ -258,17 +258,21 @@ def rank_starts(world: Sequence) -> List[int]:
     return out
 
 
-def algorithmic_bytes(T: int, K: int, H: int, in_bytes: int = 2, out_bytes: int = 2, fp8: bool = False) -> dict:
+def algorithmic_bytes(T: int, K: int, H: int, in_bytes: int = 2, out_bytes: int = 2, fp8: bool = False,
+                      stub_folded: bool = False) -> dict:
     """HBM bytes the path must move.  Index, weight and meta traffic is left out.
 
     dispatch: read ``x`` once, write ``R`` rows (plus ``4*H/128`` scale bytes per row
     for fp8); combine: read ``R`` expert rows, write ``T`` rows; stub: read the
-    dispatched rows, write ``R`` rows.
+    dispatched rows, write ``R`` rows.  ``stub_folded``: the combine reads the dispatched rows
+    themselves (fp8 bytes and scales for an fp8 dispatch) and there is no stub pass.
     """
     R = T * K
     b_d = 1 if fp8 else in_bytes
     S = 4 * H // FP8_BLOCK if fp8 else 0
     dispatch = T * H * in_bytes + R * (H * b_d + S)
+    if stub_folded:
+        return dict(dispatch=dispatch, combine=R * (H * b_d + S) + T * H * out_bytes, stub=0)
     combine = R * H * out_bytes + T * H * out_bytes
     stub = R * (H * b_d + S) + R * H * out_bytes
     return dict(dispatch=dispatch, combine=combine, stub=stub)

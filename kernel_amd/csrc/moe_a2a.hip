@@ -70,12 +70,13 @@ enum KernelId {
   KID_ROUTE_EMPTY,
   KID_FORWARD_TOKEN,
   KID_FORWARD_TILE,
+  KID_DISPATCH_FOLD,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
-    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token", "forward_tile"};
+    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token", "forward_tile", "dispatch_fold"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -779,10 +780,64 @@ static bool forward_one_launch_ok(int T, int K, int H, int max_recv, int in_type
   return forward_one_launch_form(T, K, H, max_recv, in_type, out_type, fp8_dispatch) != 0;
 }
 
+// Routing by its own launches, then dispatch and fold of each token in one kernel (dispatch_fold_kernel):
+// 16-bit rows of one element type, compact layout, stub folded in, wherever routing and dispatch
+// would be separate launches anyway.
+static bool dispatch_fold_ok(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch,
+                             int fuse_route) {
+  if (fp8_dispatch || max_recv > 0 || in_type != out_type || T < 1) return false;
+  if (option(MOE_A2A_OPT_TWO_LAUNCHES) == 1) return false;
+  return !(fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
+}
+
+static int dispatch_fold(const void* x, const int32_t* indices, const float* weights, const int32_t* slot_of_entry,
+                         void* disp, void* out, int T, int K, int E, int W, int H, int elem_type, int stub_kind,
+                         int combine_mode, hipStream_t stream) {
+  if (int rc = check_rows(x, disp, T, K, H, 8)) return rc;
+  if (!aligned16(out)) return MOE_A2A_E_ALIGN;
+  if (!indices || !weights || !slot_of_entry || !out) return MOE_A2A_E_NULL;
+  const int nvec = H / 8, E_l = E / W;
+  const bool st = streams(T, 2ll * T * K + T, H, 2, 2);
+  const RowGeom g = row_geom(nvec);
+  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
+#define DF_ARGS                                                                                                   \
+  (const uint4*)x, indices, weights, slot_of_entry, (uint4*)disp, (uint4*)out, stub_kind, E, E_l, K, nvec, g.per, \
+      g.nsplit
+#define DF4(EL, MD, KT)                                                                                            \
+  {                                                                                                                \
+    if (st) return launch(KID_DISPATCH_FOLD, dispatch_fold_kernel<EL, MD, KT, 2>, grid, block, 0, stream, DF_ARGS); \
+    return launch(KID_DISPATCH_FOLD, dispatch_fold_kernel<EL, MD, KT, 0>, grid, block, 0, stream, DF_ARGS);        \
+  }
+#define DF3(EL, MD)              \
+  {                              \
+    switch (K) {                 \
+      case 4: DF4(EL, MD, 4)     \
+      case 8: DF4(EL, MD, 8)     \
+      default: DF4(EL, MD, 0)    \
+    }                            \
+  }
+#define DF2(EL)                                                        \
+  {                                                                    \
+    if (combine_mode == MOE_A2A_COMBINE_STRICT) DF3(EL, MOE_A2A_COMBINE_STRICT) \
+    DF3(EL, MOE_A2A_COMBINE_F32)                                       \
+  }
+  if (elem_type == MOE_A2A_BF16) DF2(Bf16)
+  DF2(F16)
+#undef DF2
+#undef DF3
+#undef DF4
+#undef DF_ARGS
+}
+
 int moe_a2a_forward_launches(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch,
                              int fuse_route, int fuse_stub) {
   if (T <= 0) return 0;
   if (fuse_stub && fuse_route && forward_one_launch_ok(T, K, H, max_recv, in_type, out_type, fp8_dispatch)) return 1;
+  if (fuse_stub && dispatch_fold_ok(T, K, H, max_recv, in_type, out_type, fp8_dispatch, fuse_route)) {
+    const long long R = (long long)T * K;
+    if (R <= kRouteTilesMaxRows) return 2;
+    return ceil_div((int)std::min<long long>(R, INT32_MAX), kRouteThreads) <= kRouteFoldMaxTiles ? 3 : 4;
+  }
   const bool fused = !fp8_dispatch && (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
   int n = fused ? 1 : 2;  // routing + dispatch
   if (!fused) {
@@ -882,6 +937,13 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
     return forward_one_launch(x, indices, weights, rank_start, src_rank, T, K, E, W, H, in_type, stub_kind,
                               combine_mode, counts, offsets, slot_of_entry, src_of_slot, meta, status, disp, out,
                               (hipStream_t)stream);
+  if (T > 0 && fuse_stub && dispatch_fold_ok(T, K, H, max_recv, in_type, out_type, fp8_dispatch, fuse_route)) {
+    if (int rc = moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
+                               src_of_slot, meta, status, workspace, workspace_bytes, stream))
+      return rc;
+    return dispatch_fold(x, indices, weights, slot_of_entry, disp, out, T, K, E, W, H, in_type, stub_kind,
+                         combine_mode, (hipStream_t)stream);
+  }
   const bool fused = !fp8_dispatch && T > 0 &&
                      (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
   if (fused) {
