@@ -181,22 +181,14 @@ def lead_passes(lib, run_n, steps, gpu_step_us, torch, floor):
     return max(floor, min(lead, 2000)), launches, plain, timed
 
 
-class ForwardArgs(ctypes.Structure):
-    """Mirror of moe_a2a_forward_args in kernel_amd/csrc/bench_loop.cpp."""
-    _fields_ = ([(n, ctypes.c_void_p) for n in ("x", "indices", "weights", "rank_start")] +
-                [(n, ctypes.c_int) for n in ("src_rank", "T", "K", "E", "W", "H", "max_recv", "in_type", "out_type", "fp8_dispatch",
-                                             "stub_kind", "combine_mode", "fuse_route", "fuse_stub")] +
-                [(n, ctypes.c_void_p) for n in ("counts", "offsets", "slot_of_entry", "src_of_slot", "meta", "status",
-                                                "disp", "disp_scale", "expert_y", "out", "workspace")] +
-                [("workspace_bytes", ctypes.c_size_t), ("stream", ctypes.c_void_p)])
-
-
 def c_loop(step):
     """run(n): n back-to-back steps launched from C with the planned step's own arguments."""
     from kernel_amd import build as _build
 
     loop = ctypes.CDLL(_build.BENCH_LIB_PATH)
     loop.moe_a2a_bench_steps.restype = ctypes.c_int
+    from kernel_amd._lib import ForwardArgs
+
     loop.moe_a2a_bench_steps.argtypes = [ctypes.c_int, ctypes.POINTER(ForwardArgs), ctypes.POINTER(ForwardArgs)]
     sets = [ForwardArgs(*a) for a in step.args]
 

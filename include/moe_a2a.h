@@ -234,6 +234,29 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                     int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
                     size_t workspace_bytes, moe_a2a_stream_t stream);
 
+/*
+ * moe_a2a_forward with its arguments in a struct (same order, same meaning): a caller that repeats
+ * the call fills the struct once and patches the pointers that change, which costs a foreign-function
+ * binding one argument instead of thirty-one.
+ */
+typedef struct moe_a2a_forward_args {
+  const void* x;
+  const int32_t* indices;
+  const float* weights;
+  const int32_t* rank_start;
+  int src_rank, T, K, E, W, H, max_recv, in_type, out_type, fp8_dispatch, stub_kind, combine_mode, fuse_route,
+      fuse_stub;
+  int32_t *counts, *offsets, *slot_of_entry, *src_of_slot, *meta, *status;
+  void* disp;
+  float* disp_scale;
+  void* expert_y;
+  void* out;
+  void* workspace;
+  size_t workspace_bytes;
+  moe_a2a_stream_t stream;
+} moe_a2a_forward_args;
+int moe_a2a_forward_packed(const moe_a2a_forward_args* args);
+
 /* Kernel launches moe_a2a_forward issues for this shape and these switches (host logic only). */
 int moe_a2a_forward_launches(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch,
                              int fuse_route, int fuse_stub);

@@ -57,6 +57,20 @@ PROTOTYPES = {
     "moe_a2a_kernel_name": (C.c_char_p, [_int]),
 }
 
+
+
+class ForwardArgs(C.Structure):
+    """``moe_a2a_forward_args`` of include/moe_a2a.h."""
+    _fields_ = ([(n, C.c_void_p) for n in ("x", "indices", "weights", "rank_start")] +
+                [(n, C.c_int) for n in ("src_rank", "T", "K", "E", "W", "H", "max_recv", "in_type", "out_type",
+                                        "fp8_dispatch", "stub_kind", "combine_mode", "fuse_route", "fuse_stub")] +
+                [(n, C.c_void_p) for n in ("counts", "offsets", "slot_of_entry", "src_of_slot", "meta", "status", "disp",
+                                           "disp_scale", "expert_y", "out", "workspace")] +
+                [("workspace_bytes", C.c_size_t), ("stream", C.c_void_p)])
+
+
+PROTOTYPES["moe_a2a_forward_packed"] = (_int, [C.POINTER(ForwardArgs)])
+
 _lib = None
 
 

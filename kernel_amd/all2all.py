@@ -17,6 +17,8 @@ torch is used for device memory and the current stream only.
 """
 from __future__ import annotations
 
+import collections
+import ctypes
 import dataclasses
 from typing import Optional, Sequence
 
@@ -43,12 +45,13 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
-def _stream() -> int:
-    """Handle of torch's current stream on the current device.  The raw query is one C call; the
-    public one builds a Stream object and resolves the device twice (8 us of a 19 us forward)."""
+def _stream(device_index: Optional[int] = None) -> int:
+    """Handle of torch's current stream on the current device (or the one named).  The raw query is
+    one C call; the public one builds a Stream object and resolves the device twice (8 us of a 19 us
+    forward)."""
     if _raw_stream is not None:
-        return _raw_stream(torch.cuda.current_device())
-    return torch.cuda.current_stream().cuda_stream
+        return _raw_stream(torch.cuda.current_device() if device_index is None else device_index)
+    return torch.cuda.current_stream(device_index).cuda_stream
 
 
 def _require_gpu(t: torch.Tensor, name: str) -> None:
@@ -111,6 +114,7 @@ class HipAllToAll:
     """MoE dispatch / expert stub / combine on one MI355X."""
 
     META_DIM = META_DIM
+    MAX_CACHED_SHAPES = 8  # token counts whose buffers are kept (two sets each)
 
     def __init__(self, cfg: MoEConfig, rank: int, world_size: int, stub_kind: int = STUB_OWNER_RANK,
                  combine_mode: int = COMBINE_STRICT, fp8_dispatch: bool = False, fuse_route: bool = True,
@@ -134,7 +138,7 @@ class HipAllToAll:
         self.fuse_stub = fuse_stub
         self.lib = _lib.load()
         self._fused_max_rows = self.lib.moe_a2a_fused_max_rows()
-        self._bufs = {}
+        self._bufs = collections.OrderedDict()  # (T, device) -> two buffer sets; least recently used goes first
 
     # ---- buffers ---------------------------------------------------------------------
     def _buffers(self, T: int, device, advance: bool = False) -> dict:
@@ -145,15 +149,26 @@ class HipAllToAll:
         step never writes what the step before it read; it also means the result of a call
         stays valid until the second-next call.
         """
-        key = (T, str(device))
+        key = (T, device)
         ring = self._bufs.get(key)
         if ring is None:
+            while len(self._bufs) >= self.MAX_CACHED_SHAPES:  # a caller with many token counts keeps the recent ones
+                self._bufs.popitem(last=False)
             ring = self._bufs[key] = dict(sets=[None, None], cur=0)
+        else:
+            self._bufs.move_to_end(key)
         if advance:
             ring["cur"] ^= 1
         b = ring["sets"][ring["cur"]]
         if b is not None:
             return b
+        # both sets of a new shape are allocated together, so that the second call with this shape
+        # does not meet an allocation either
+        for i in (0, 1):
+            ring["sets"][i] = self._allocate(T, device)
+        return ring["sets"][ring["cur"]]
+
+    def _allocate(self, T: int, device) -> dict:
         cfg = self.cfg
         K, H, E = cfg.experts_per_token, cfg.hidden_dim, cfg.num_experts
         R = T * K
@@ -168,7 +183,9 @@ class HipAllToAll:
             status=torch.zeros(1, **i32),
             workspace=torch.empty(max(self.lib.moe_a2a_workspace_bytes(T, K, E), 256), dtype=torch.uint8,
                                   device=device),
-            expert_y=torch.empty(rows, H, dtype=cfg.out_dtype, device=device),
+            # the stub's output rows exist only where the stub is a launch of its own (expert_stub
+            # allocates them on first use otherwise)
+            expert_y=None if self.fuse_stub else torch.empty(rows, H, dtype=cfg.out_dtype, device=device),
             out=torch.empty(T, H, dtype=cfg.out_dtype, device=device),
         )
         if self.fp8_dispatch:
@@ -177,7 +194,6 @@ class HipAllToAll:
         else:
             b["disp_x"] = torch.empty(rows, H, dtype=cfg.in_dtype, device=device)
             b["disp_scale"] = None
-        ring["sets"][ring["cur"]] = b
         return b
 
     def release_buffers(self) -> None:
@@ -234,7 +250,10 @@ class HipAllToAll:
         """all2all/reference.py:262 on the compact rows -> ``expert_y[R,H]`` out_dtype."""
         cfg = self.cfg
         R, H = d.num_rows, d.disp_x.shape[1]
-        y = self._buffers(d.num_tokens, d.disp_x.device)["expert_y"]
+        b = self._buffers(d.num_tokens, d.disp_x.device)
+        if b["expert_y"] is None:
+            b["expert_y"] = torch.empty(d.disp_x.shape[0], H, dtype=cfg.out_dtype, device=d.disp_x.device)
+        y = b["expert_y"]
         in_type = _lib.BF16 if d.disp_scale is not None else _elem(d.disp_x.dtype)
         rows = d.slot_of_entry if d.max_recv > 0 else None  # padded: only rows that hold an entry
         _lib.check(self.lib.moe_a2a_stub(_ptr(d.disp_x), _ptr(d.disp_scale), _ptr(d.meta), _ptr(rows), in_type,
@@ -354,11 +373,14 @@ class HipAllToAll:
 
     def _check_inputs(self, x, indices, weights, rank_start) -> None:
         cfg = self.cfg
-        for name, t in (("x", x), ("indices", indices), ("weights", weights)):
-            _require_gpu(t, name)
+        if not (x.is_cuda and indices.is_cuda and weights.is_cuda and x.is_contiguous() and indices.is_contiguous()
+                and weights.is_contiguous()):
+            for name, t in (("x", x), ("indices", indices), ("weights", weights)):
+                _require_gpu(t, name)  # raises, naming the tensor
         T, H = x.shape
         K = cfg.experts_per_token
-        if (H != cfg.hidden_dim or tuple(indices.shape) != (T, K) or tuple(weights.shape) != (T, K)
+        si, sw = indices.shape, weights.shape
+        if (H != cfg.hidden_dim or len(si) != 2 or si[0] != T or si[1] != K or len(sw) != 2 or sw[0] != T or sw[1] != K
                 or x.dtype != cfg.in_dtype or indices.dtype != torch.int32 or weights.dtype != torch.float32):
             raise ValueError("x / indices / weights do not match the MoEConfig")
         if rank_start is not None:
@@ -386,19 +408,28 @@ class HipAllToAll:
             if out.dtype != cfg.out_dtype or out.dim() != 2 or out.shape[0] < T or out.shape[1] != cfg.hidden_dim:
                 raise ValueError("out must be out_dtype[>=T,H]")
         b = self._buffers(T, x.device, advance=True)
-        # the argument list of a buffer set is built once; a call patches the caller's pointers in
-        args = b.get("_args")
-        if args is None:
-            args = b["_args"] = list(self._forward_args(b, x, indices, weights, rank_start, 0))
+        # the argument struct of a buffer set is built once; a call patches the caller's pointers in
+        a = b.get("_args")
+        if a is None:
+            a = b["_args"] = _lib.ForwardArgs(*self._forward_args(b, x, indices, weights, rank_start, 0))
+            b["_argp"] = ctypes.pointer(a)
             b["_record"] = self._record(b, T)
-        args[0], args[1], args[2] = x.data_ptr(), indices.data_ptr(), weights.data_ptr()
-        args[3] = None if rank_start is None else rank_start.data_ptr()
-        args[14], args[15] = self.stub_kind, self.combine_mode
-        args[16] = 2 if self.fuse_route == "always" else int(bool(self.fuse_route))
-        args[17] = int(self.fuse_stub)
-        args[27] = b["out"].data_ptr() if out is None else out.data_ptr()
-        args[30] = _stream()
-        _lib.check(self.lib.moe_a2a_forward(*args), "moe_a2a_forward")
+        a.x, a.indices, a.weights = x.data_ptr(), indices.data_ptr(), weights.data_ptr()
+        a.out = b["out"].data_ptr() if out is None else out.data_ptr()
+        # what rarely changes between two calls is written only when it does (a field of a foreign
+        # struct costs a quarter of a microsecond to set)
+        rs = None if rank_start is None else rank_start.data_ptr()
+        st = _stream(x.device.index)
+        switches = (rs, st, self.stub_kind, self.combine_mode, self.fuse_route, self.fuse_stub)
+        if b.get("_switches") != switches:
+            b["_switches"] = switches
+            a.rank_start, a.stream = rs, st
+            a.stub_kind, a.combine_mode = self.stub_kind, self.combine_mode
+            a.fuse_route = 2 if self.fuse_route == "always" else int(bool(self.fuse_route))
+            a.fuse_stub = int(self.fuse_stub)
+        rc = self.lib.moe_a2a_forward_packed(b["_argp"])
+        if rc:
+            raise _lib.MoeA2AError(rc, "moe_a2a_forward")
         self.last = b["_record"]
         return b["out"] if out is None else out
 
@@ -421,14 +452,16 @@ class HipAllToAll:
         args = [self._forward_args(b, x, indices, weights, rank_start, st) for b in sets]
         outs = [b["out"] for b in sets]
         records = [self._record(b, T) for b in sets]
-        fn = self.lib.moe_a2a_forward
-        keep = (x, indices, weights, rank_start)  # the raw pointers above must stay valid
+        fn = self.lib.moe_a2a_forward_packed
+        structs = [_lib.ForwardArgs(*a) for a in args]
+        ptrs = [ctypes.pointer(st_) for st_ in structs]
+        keep = (x, indices, weights, rank_start, structs)  # the raw pointers above must stay valid
         state = [0]
 
         def step() -> torch.Tensor:
             i = state[0]
             state[0] = i ^ 1
-            rc = fn(*args[i])
+            rc = fn(ptrs[i])
             if rc:
                 raise _lib.MoeA2AError(rc, "moe_a2a_forward")
             self.last = records[i]

@@ -101,7 +101,13 @@ struct F16 {
   static __device__ __forceinline__ float hi(uint32_t u) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(u >> 16));
   }
+  // Two roundings, as torch does them: the caller's f32 arithmetic rounds to f32, the conversion
+  // rounds that f32 to f16.  The empty asm hides where a and b come from: left to itself the
+  // compiler merges a preceding multiply or add into v_fma_mixlo_f16, which rounds the exact
+  // product or sum ONCE to f16 and gives a different last bit in a fraction of a percent of the
+  // values (seen against the oracle on fp8 rows, where the f32 product is rarely exact).
   static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    asm("" : "+v"(a), "+v"(b));
     uint32_t l = __builtin_bit_cast(uint16_t, (_Float16)a);
     uint32_t h = __builtin_bit_cast(uint16_t, (_Float16)b);
     return l | (h << 16);
@@ -785,9 +791,48 @@ static bool forward_one_launch_ok(int T, int K, int H, int max_recv, int in_type
 // would be separate launches anyway.
 static bool dispatch_fold_ok(int T, int K, int H, int max_recv, int in_type, int out_type, int fp8_dispatch,
                              int fuse_route) {
-  if (fp8_dispatch || max_recv > 0 || in_type != out_type || T < 1) return false;
+  if (max_recv > 0 || in_type != out_type || T < 1) return false;
   if (option(MOE_A2A_OPT_TWO_LAUNCHES) == 1) return false;
+  // The fp8 dispatch is always routed by a launch of its own.  The fold behind it pays while the rows
+  // stay in the caches (one launch boundary less); at streaming volumes the two separate kernels move
+  // the same bytes about 1 % faster (120.0 against 118.8 us at 16384 tokens, top-8, H = 7168).
+  if (fp8_dispatch) return !streams(T, 2ll * T * K, H, 2, 1);
   return !(fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
+}
+
+static int dispatch_fold_fp8(const void* x, const int32_t* indices, const float* weights,
+                             const int32_t* slot_of_entry, void* disp_q, float* disp_scale, void* out, int T, int K,
+                             int E, int W, int H, int elem_type, int stub_kind, int combine_mode, int pow2,
+                             hipStream_t stream) {
+  if (int rc = check_rows(x, disp_q, T, K, H, MOE_A2A_FP8_BLOCK)) return rc;
+  if (!aligned16(out)) return MOE_A2A_E_ALIGN;
+  if (!indices || !weights || !slot_of_entry || !disp_scale || !out) return MOE_A2A_E_NULL;
+  const int nblk = H / MOE_A2A_FP8_BLOCK, E_l = E / W;
+  const RowGeom g = row_geom(nblk * 8, 8);  // cache-resident volumes only: see dispatch_fold_ok
+  dim3 grid((unsigned)T * g.nsplit), block(g.threads);
+#define DF8_ARGS                                                                                                  \
+  (const uint4*)x, indices, weights, slot_of_entry, (uint4*)disp_q, disp_scale, (uint4*)out, stub_kind, E, E_l, K, \
+      nblk, g.per, g.nsplit, pow2
+#define DF84(EL, MD, KT) \
+  return launch(KID_DISPATCH_FOLD, dispatch_fold_fp8_kernel<EL, MD, KT, 0>, grid, block, 0, stream, DF8_ARGS);
+#define DF83(EL, MD)             \
+  {                              \
+    switch (K) {                 \
+      case 8: DF84(EL, MD, 8)    \
+      default: DF84(EL, MD, 0)   \
+    }                            \
+  }
+#define DF82(EL)                                                        \
+  {                                                                     \
+    if (combine_mode == MOE_A2A_COMBINE_STRICT) DF83(EL, MOE_A2A_COMBINE_STRICT) \
+    DF83(EL, MOE_A2A_COMBINE_F32)                                       \
+  }
+  if (elem_type == MOE_A2A_BF16) DF82(Bf16)
+  DF82(F16)
+#undef DF82
+#undef DF83
+#undef DF84
+#undef DF8_ARGS
 }
 
 static int dispatch_fold(const void* x, const int32_t* indices, const float* weights, const int32_t* slot_of_entry,
@@ -941,6 +986,9 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
     if (int rc = moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
                                src_of_slot, meta, status, workspace, workspace_bytes, stream))
       return rc;
+    if (fp8_dispatch)
+      return dispatch_fold_fp8(x, indices, weights, slot_of_entry, disp, disp_scale, out, T, K, E, W, H, in_type,
+                               stub_kind, combine_mode, fp8_dispatch == 2, (hipStream_t)stream);
     return dispatch_fold(x, indices, weights, slot_of_entry, disp, out, T, K, E, W, H, in_type, stub_kind,
                          combine_mode, (hipStream_t)stream);
   }
@@ -971,6 +1019,15 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
     return rc;
   return combine_impl(expert_y, weights, slot_of_entry, combine_mode, out_type, out, T, K, H,
                       (long long)T * K * H * (fp8_dispatch ? 1 : 2), stream);
+}
+
+int moe_a2a_forward_packed(const moe_a2a_forward_args* a) {
+  if (!a) return MOE_A2A_E_NULL;
+  return moe_a2a_forward(a->x, a->indices, a->weights, a->rank_start, a->src_rank, a->T, a->K, a->E, a->W, a->H,
+                         a->max_recv, a->in_type, a->out_type, a->fp8_dispatch, a->stub_kind, a->combine_mode,
+                         a->fuse_route, a->fuse_stub, a->counts, a->offsets, a->slot_of_entry, a->src_of_slot, a->meta,
+                         a->status, a->disp, a->disp_scale, a->expert_y, a->out, a->workspace, a->workspace_bytes,
+                         a->stream);
 }
 
 // Launch of the 256 x 256 kernel; x_scale != nullptr selects fp8 rows of x, w_scale != nullptr

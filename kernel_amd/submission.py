@@ -18,7 +18,7 @@ _instances = {}
 
 def _instance(cfg, rank: int, world_size: int, device, stub_kind: int, combine_mode: int) -> HipAllToAll:
     key = (cfg.num_experts, cfg.experts_per_token, cfg.hidden_dim, cfg.in_dtype, cfg.out_dtype, rank, world_size,
-           str(device), stub_kind, combine_mode)
+           device, stub_kind, combine_mode)
     ata = _instances.get(key)
     if ata is None:
         if len(_instances) > 64:
@@ -35,15 +35,27 @@ def custom_kernel(data, stub_kind: int = STUB_OWNER_RANK, combine_mode: int = CO
     x = rank_data.x
     if not x.is_cuda:
         raise RuntimeError("custom_kernel needs its inputs on the GPU: there is no CPU implementation")
-    ata = _instance(cfg, rank, world_size, x.device, stub_kind, combine_mode)
+    # the instance found for this cfg object last time is kept on it (a harness calls with the same
+    # cfg many times); the key of the full look-up is rebuilt only for a new object or other switches
+    slot = getattr(cfg, "__dict__", None)
+    memo = slot.get("_hip_a2a") if slot is not None else None
+    if memo is not None and memo[0] == (rank, world_size, x.device, stub_kind, combine_mode):
+        ata = memo[1]
+    else:
+        ata = _instance(cfg, rank, world_size, x.device, stub_kind, combine_mode)
+        if slot is not None:
+            slot["_hip_a2a"] = ((rank, world_size, x.device, stub_kind, combine_mode), ata)
     T = x.shape[0]
     # the caller owns its result (eval.py deletes it after each run): the combine writes straight
     # into a fresh tensor instead of one of the reused buffers
-    y = torch.empty(T, cfg.hidden_dim, dtype=cfg.out_dtype, device=x.device)
-    args = (x.contiguous(), rank_data.indices.contiguous(), rank_data.weights.contiguous())
+    y = torch.empty((T, cfg.hidden_dim), dtype=cfg.out_dtype, device=x.device)
+    idx, w = rank_data.indices, rank_data.weights
+    if not (x.is_contiguous() and idx.is_contiguous() and w.is_contiguous()):
+        x, idx, w = x.contiguous(), idx.contiguous(), w.contiguous()
     if x.device.index == torch.cuda.current_device():  # the usual case: no device switch to pay for
-        ata.forward(*args, out=y)
+        ata.forward(x, idx, w, out=y)
     else:
         with torch.cuda.device(x.device):
-            ata.forward(*args, out=y)
-    return y[: rank_data.num_tokens]
+            ata.forward(x, idx, w, out=y)
+    n = rank_data.num_tokens
+    return y if n == T else y[:n]

@@ -386,6 +386,41 @@ def test_one_launch_forward_equals_the_oracle_and_the_two_launch_form(gpu_device
     assert lib.moe_a2a_kernel_name(ids[0]) in (b"forward_token", b"forward_tile")
 
 
+@pytest.mark.parametrize("W,E,K,H,tokens", [
+    (1, 8, 2, 256, [64]),
+    (8, 256, 8, 7168, [40, 0, 3, 0, 17, 0, 0, 1]),
+    (2, 16, 3, 384, [100, 37]),          # three 128-column blocks, K without a specialised fold
+    (4, 32, 4, 4096, [300, 0, 123, 9]),
+])
+@pytest.mark.parametrize("fp8", [True, "pow2"], ids=["f32scales", "pow2scales"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("mode", [C.COMBINE_STRICT, C.COMBINE_F32], ids=["strict", "f32"])
+def test_forward_with_fp8_dispatch_and_folded_stub(gpu_device, options, W, E, K, H, tokens, fp8, dtype, mode):
+    """forward with an fp8 dispatch and the stub folded in quantises, stores and folds a token in one
+    kernel behind the routing launch: rows, scales and output bit for bit those of the oracle and of
+    the separate dispatch_fp8 + stub_combine launches."""
+    g = torch.Generator().manual_seed(sum(tokens) + E + K)
+    cfg = C.MoEConfig(E, K, H, max(tokens) + 1, dtype, dtype)
+    world = []
+    for n in tokens:
+        idx = (torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(n)]).to(torch.int32) if n
+               else torch.empty(0, K, dtype=torch.int32))
+        world.append(C.RankData(n, idx, torch.rand(n, K, generator=g), torch.randn(n, H, generator=g).to(dtype)))
+    x, idx, w, rs = concat_world(world, gpu_device)
+    want = V.run_world(cfg, world, stub_kind=C.STUB_EXPERT_FRACTION, fp8=True, combine_mode=mode, pow2=fp8 == "pow2")
+    for two in (1, 0):
+        options.set("TWO_LAUNCHES", two)  # 1: routing, dispatch_fp8 and stub_combine as separate launches
+        ata = HipAllToAll(cfg, 0, W, stub_kind=C.STUB_EXPERT_FRACTION, combine_mode=mode, fp8_dispatch=fp8,
+                          fuse_stub=True)
+        for _ in range(2):
+            y = ata.forward(x, idx, w, rs)
+        torch.cuda.synchronize()
+        d = ata.last
+        for key, val in (("counts", d.counts), ("slot_of_entry", d.slot_of_entry), ("meta", d.meta),
+                         ("disp_x", d.disp_x), ("disp_scale", d.disp_scale), ("y", y)):
+            assert_same(f"{key} ({'separate launches' if two else 'one kernel'})", val, want[key])
+
+
 @pytest.mark.parametrize("name", GOLDEN_CASES)
 @pytest.mark.parametrize("fuse_route", ["always", False])
 def test_padded_layout_is_the_reference_dispatch_return_value(gpu_device, name, fuse_route):
