@@ -14,6 +14,9 @@
 //   dispatch_fp8       same copy with e4m3fn quantisation per 128 columns
 //   stub_*             expert stand-in, one factor per row
 //   combine / stub_combine   gather K rows per token, weighted sum
+//   forward_token / forward_tile   the whole path of a token (routing, dispatch, stub, weighted sum)
+//                      in one launch: a workgroup reads back the rows it stored itself
+//   dispatch_fold      dispatch, stub and weighted sum of a token behind a routing of its own
 //   expert_gemm        y[rows of e] = x[rows of e] * W_e^T, 128 x 128 tiles (short segments)
 //   expert_gemm_wide   the same on 256 x 256 tiles, software-pipelined; 16-bit or fp8 rows
 #include <hip/hip_runtime.h>
@@ -1030,248 +1033,7 @@ int moe_a2a_forward_packed(const moe_a2a_forward_args* a) {
                          a->stream);
 }
 
-// Launch of the 256 x 256 kernel; x_scale != nullptr selects fp8 rows of x, w_scale != nullptr
-// block-quantised weights.
-static int launch_gemm_wide(const void* x, const float* x_scale, const void* weights, const float* w_scale,
-                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
-                            hipStream_t stream, bool mx = false) {
-  const int ntile_n = ceil_div(N, kWideN);
-  const long long mtiles = (long long)R / kWideM + E;  // every expert may end with a partly filled tile
-  if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-  dim3 grid((unsigned)(mtiles * ntile_n)), block(kWideThreads);
-  // the kernels need more dynamic LDS than the 64 KB default: raised once per device (the
-  // attribute belongs to the device's copy of the function); racing first calls only repeat it
-  static std::atomic<bool> lds_raised[kMaxDevices];
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
-  if (dev < 0 || dev >= kMaxDevices) return MOE_A2A_E_STATE;
-  if (!lds_raised[dev].load(std::memory_order_acquire)) {
-    const void* kernels[10] = {(const void*)expert_gemm_wide_kernel<Bf16, false, false, true>,
-                              (const void*)expert_gemm_wide_kernel<F16, false, false, true>,
-                              (const void*)expert_gemm_wide_kernel<Bf16, false, false>,
-                              (const void*)expert_gemm_wide_kernel<F16, false, false>,
-                              (const void*)expert_gemm_wide_kernel<Bf16, true, false>,
-                              (const void*)expert_gemm_wide_kernel<F16, true, false>,
-                              (const void*)expert_gemm_wide_kernel<Bf16, false, true>,
-                              (const void*)expert_gemm_wide_kernel<F16, false, true>,
-                              (const void*)expert_gemm_wide_kernel<Bf16, true, true>,
-                              (const void*)expert_gemm_wide_kernel<F16, true, true>};
-    for (const void* k : kernels) {
-      hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes);
-      if (e != hipSuccess) return (int)e;
-    }
-    lds_raised[dev].store(true, std::memory_order_release);
-  }
-#define CALL_WIDE(ET, AF, BF)                                                                                  \
-  return launch(KID_EXPERT_GEMM_WIDE, expert_gemm_wide_kernel<ET, AF, BF>, grid, block, kWideLdsBytes, stream, \
-                (const uint4*)x, x_scale, (const uint4*)weights, w_scale, offsets, (uint16_t*)y, E, Kd, N,     \
-                max_recv, ntile_n)
-#define CALL_WIDE_E(ET)                  \
-  {                                      \
-    if (mx)                                                                                                    \
-      return launch(KID_EXPERT_GEMM_MX, expert_gemm_wide_kernel<ET, false, false, true>, grid, block,          \
-                    kWideLdsBytes, stream, (const uint4*)x, x_scale, (const uint4*)weights, w_scale, offsets,  \
-                    (uint16_t*)y, E, Kd, N, max_recv, ntile_n);                                                \
-    if (x_scale && w_scale) CALL_WIDE(ET, true, true);  \
-    if (x_scale) CALL_WIDE(ET, true, false);            \
-    if (w_scale) CALL_WIDE(ET, false, true);            \
-    CALL_WIDE(ET, false, false);                        \
-  }
-  if (elem_type == MOE_A2A_BF16) CALL_WIDE_E(Bf16);
-  CALL_WIDE_E(F16);
-#undef CALL_WIDE_E
-#undef CALL_WIDE
-}
-
-int moe_a2a_expert_gemm(const void* x, const void* weights, const int32_t* offsets, void* y, int R, int E, int Kd,
-                        int N, int max_recv, int elem_type, moe_a2a_stream_t stream_) {
-  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
-  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < kGemmK || Kd % kGemmK != 0 || N < 8 || N % 8 != 0 ||
-      max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8)
-    return MOE_A2A_E_SHAPE;
-  if (R == 0) return 0;
-  if (!x || !weights || !offsets || !y) return MOE_A2A_E_NULL;
-  if (!aligned16(x) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
-  hipStream_t stream = (hipStream_t)stream_;
-  // Long segments take the 256 x 256 kernel: with fewer than 256 rows per expert on average most
-  // of its tiles would be half empty.  the option MOE_A2A_OPT_GEMM_TILE = 32 | 128 | 256 overrides.
-  // Short segments (a decode step) take the 32 x 256 kernel, which streams the weights.
-  bool wide = (long long)R >= 256ll * E && N >= kWideN;
-  bool skinny = (long long)R <= 32ll * E;
-  if (const int forced = option(MOE_A2A_OPT_GEMM_TILE)) {
-    wide = forced == 256;
-    skinny = forced == 32;
-  }
-  if (Kd % kSkinnyK != 0) skinny = false;  // its K slabs are 128 wide; the 128 x 128 kernel takes the rest
-  if (wide) return launch_gemm_wide(x, nullptr, weights, nullptr, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
-  if (skinny) {
-    const int ntile_n = ceil_div(N, kSkinnyN);
-    const long long mtiles = (long long)R / kSkinnyM + E;
-    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-    dim3 grid((unsigned)(mtiles * ntile_n)), block(kSkinnyThreads);
-    if (elem_type == MOE_A2A_BF16)
-      return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_skinny_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
-                    (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-    return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_skinny_kernel<F16>, grid, block, 0, stream, (const uint4*)x,
-                  (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-  }
-  const int ntile_n = ceil_div(N, kGemmN);
-  // worst case of m-tiles: every expert ends with a partly filled tile
-  const long long mtiles = (long long)R / kGemmM + E;
-  if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-  dim3 grid((unsigned)(mtiles * ntile_n)), block(kGemmThreads);
-  if (elem_type == MOE_A2A_BF16)
-    return launch(KID_EXPERT_GEMM, expert_gemm_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
-                  (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-  return launch(KID_EXPERT_GEMM, expert_gemm_kernel<F16>, grid, block, 0, stream, (const uint4*)x,
-                (const uint4*)weights, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-}
-
-int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* weights, const int32_t* offsets,
-                            void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
-                            moe_a2a_stream_t stream_) {
-  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
-  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 || N < 8 ||
-      N % 8 != 0 || max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8)
-    return MOE_A2A_E_SHAPE;
-  if (R == 0) return 0;
-  if (!x_q || !x_scale || !weights || !offsets || !y) return MOE_A2A_E_NULL;
-  if (!aligned16(x_q) || !aligned16(weights) || !aligned16(y)) return MOE_A2A_E_ALIGN;
-  return launch_gemm_wide(x_q, x_scale, weights, nullptr, offsets, y, R, E, Kd, N, max_recv, elem_type,
-                          (hipStream_t)stream_);
-}
-
-int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q, const float* w_scale,
-                           const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
-                           moe_a2a_stream_t stream_) {
-  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
-  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 ||
-      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0 ||
-      (long long)max_recv * E > (long long)INT32_MAX / 8)
-    return MOE_A2A_E_SHAPE;
-  if (R == 0) return 0;
-  if (!x || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
-  if (!aligned16(x) || !aligned16(w_q) || !aligned16(y)) return MOE_A2A_E_ALIGN;
-  hipStream_t stream = (hipStream_t)stream_;
-  // A decode step streams the weights (32-row tiles); longer segments multiply fp8 by fp8 when the
-  // rows are fp8, else on the 256 x 256 kernel, which dequantises the weights on their way into LDS
-  // (it needs N >= 256).  The option MOE_A2A_OPT_GEMM_TILE = 32 | 128 | 256 forces one where it applies.
-  enum { kStream, kBothFp8, kDequant } kernel;
-  if ((long long)R <= 32ll * E) kernel = kStream;
-  else if (x_scale) kernel = kBothFp8;
-  else kernel = N >= kWideN ? kDequant : kStream;
-  if (const int tile = option(MOE_A2A_OPT_GEMM_TILE)) {
-    if (tile == 32) kernel = kStream;
-    if (tile == 128 && x_scale) kernel = kBothFp8;
-    if (tile == 256 && N >= kWideN) kernel = kDequant;
-  }
-  if (kernel == kDequant)
-    return launch_gemm_wide(x, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream);
-  if (kernel == kBothFp8) {
-    // both operands fp8: the bytes go to the matrix cores as they are.  128 x 128 tiles: the
-    // 128 x 256 form of the kernel (one workgroup of eight waves per CU) measured slower, 1160
-    // against 1140 us at 128 rows per expert and 1030 against 920 us at 512.
-    constexpr int tn = 128;
-    const int ntile_n = N / tn;
-    // worst case of m-tiles (every expert ends with a partly filled one), an eighth of them per XCD
-    const long long mtiles = ((long long)R / kF8M + E + kXcds - 1) / kXcds * kXcds;
-    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-    dim3 grid((unsigned)(mtiles * ntile_n)), block(2 * tn);
-    if (elem_type == MOE_A2A_BF16)
-      return launch(KID_EXPERT_GEMM_F8, expert_gemm_f8_kernel<Bf16, tn>, grid, block, 0, stream, (const uint4*)x,
-                    x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-    return launch(KID_EXPERT_GEMM_F8, expert_gemm_f8_kernel<F16, tn>, grid, block, 0, stream, (const uint4*)x,
-                  x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-  }
-  if (x_scale && option(MOE_A2A_OPT_GEMM_STAGED) != 1) {
-    // both operands fp8: the bytes stream memory -> LDS -> matrix cores, nothing is decoded
-    const int ntile_n = N / kF8sN;
-    const long long mtiles = (long long)R / kF8sM + E;
-    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-    dim3 grid((unsigned)(mtiles * ntile_n)), block(kF8sThreads);
-    if (elem_type == MOE_A2A_BF16)
-      return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_f8s_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
-                    x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-    return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_f8s_kernel<F16>, grid, block, 0, stream, (const uint4*)x, x_scale,
-                  (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-  }
-  if (!x_scale && option(MOE_A2A_OPT_GEMM_STAGED) != 1) {
-    // 16-bit rows: the slabs stream memory -> LDS, the weight bytes become 16-bit fragments in registers
-    const int ntile_n = N / kF8sN;
-    const long long mtiles = (long long)R / kF8sM + E;
-    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-    dim3 grid((unsigned)(mtiles * ntile_n)), block(kF8sThreads);
-    if (elem_type == MOE_A2A_BF16)
-      return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_q8s_kernel<Bf16>, grid, block, 0, stream, (const uint4*)x,
-                    (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-    return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_q8s_kernel<F16>, grid, block, 0, stream, (const uint4*)x,
-                  (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, ntile_n);
-  }
-  const int ntile_n = N / 128;
-  const long long mtiles = (long long)R / kSkinnyM + E;
-  if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-  dim3 grid((unsigned)(mtiles * ntile_n)), block(kSkinnyThreads);
-#define CALL_SKQ(ET, AF)                                                                                        \
-  return launch(KID_EXPERT_GEMM_SKINNY, expert_gemm_skinny_q_kernel<ET, AF>, grid, block, 0, stream,       \
-                (const uint4*)x, x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv, \
-                ntile_n)
-  if (elem_type == MOE_A2A_BF16) {
-    if (x_scale) CALL_SKQ(Bf16, true);
-    CALL_SKQ(Bf16, false);
-  }
-  if (x_scale) CALL_SKQ(F16, true);
-  CALL_SKQ(F16, false);
-#undef CALL_SKQ
-}
-
-int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w_q, const float* w_scale,
-                            const int32_t* offsets, void* y, int R, int E, int Kd, int N, int max_recv, int elem_type,
-                            moe_a2a_stream_t stream_) {
-  if (!known_type(elem_type)) return MOE_A2A_E_DTYPE;
-  if (R < 0 || E < 1 || E > MOE_A2A_MAX_EXPERTS || Kd < MOE_A2A_FP8_BLOCK || Kd % MOE_A2A_FP8_BLOCK != 0 ||
-      N < MOE_A2A_FP8_BLOCK || N % MOE_A2A_FP8_BLOCK != 0 || max_recv < 0 ||
-      (long long)max_recv * E > (long long)INT32_MAX / 8)
-    return MOE_A2A_E_SHAPE;
-  if (R == 0) return 0;
-  if (!x_q || !x_scale || !w_q || !w_scale || !offsets || !y) return MOE_A2A_E_NULL;
-  if (!aligned16(x_q) || !aligned16(w_q) || !aligned16(y)) return MOE_A2A_E_ALIGN;
-  // A decode step (R <= 32 E) is bound by the weight bytes: moe_a2a_expert_gemm_q8 streams them, and
-  // powers of two are f32 scales like any other.  Otherwise 256 x 256 tiles with the scales as block
-  // exponents: slabs sent memory -> LDS directly when Kd is a multiple of 256 (measured against the
-  // kernel that folds f32 scales on the vector units: 951 / 1140 us at 128 rows per expert,
-  // 7168 -> 2048; 735 / 923 us and 2562 / 3420 us at 512 rows per expert, 4096 -> 2048 and -> 7168),
-  // the register-staged loop for other Kd on long segments (3109 us in the last case), the folding
-  // kernel for what is left.  The option MOE_A2A_OPT_GEMM_TILE = 32 | 128 forces the streaming / the folding kernel,
-  // 256 the tiles; MOE_A2A_OPT_GEMM_STAGED = 1 the register-staged loop.
-  enum { kStream, kFold, kTilesDirect, kTilesStaged } kernel;
-  const bool staged_only = Kd % 256 != 0 || option(MOE_A2A_OPT_GEMM_STAGED) == 1;
-  if ((long long)R <= 32ll * E) kernel = kStream;
-  else if (!staged_only) kernel = kTilesDirect;
-  else kernel = (long long)R >= 256ll * E ? kTilesStaged : kFold;
-  if (const int tile = option(MOE_A2A_OPT_GEMM_TILE)) {
-    if (tile == 32) kernel = kStream;
-    if (tile == 128) kernel = kFold;
-    if (tile == 256) kernel = staged_only ? kTilesStaged : kTilesDirect;
-  }
-  if (kernel == kStream || kernel == kFold)  // the same environment variable picks between the two there
-    return moe_a2a_expert_gemm_q8(x_q, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type, stream_);
-  if (kernel == kTilesDirect) {
-    const int ntile_n = ceil_div(N, 256);
-    // worst case of m-tiles (every expert ends with a partly filled one), an eighth of them per XCD
-    const long long mtiles = ((long long)R / 256 + E + kXcds - 1) / kXcds * kXcds;
-    if (mtiles * ntile_n > INT32_MAX) return MOE_A2A_E_SHAPE;
-    dim3 grid((unsigned)(mtiles * ntile_n)), block(kMxdThreads);
-    if (elem_type == MOE_A2A_BF16)
-      return launch(KID_EXPERT_GEMM_MX, expert_gemm_mxd_kernel<Bf16>, grid, block, 0, (hipStream_t)stream_,
-                    (const uint4*)x_q, x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv,
-                    ntile_n);
-    return launch(KID_EXPERT_GEMM_MX, expert_gemm_mxd_kernel<F16>, grid, block, 0, (hipStream_t)stream_,
-                  (const uint4*)x_q, x_scale, (const uint4*)w_q, w_scale, offsets, (uint16_t*)y, E, Kd, N, max_recv,
-                  ntile_n);
-  }
-  return launch_gemm_wide(x_q, x_scale, w_q, w_scale, offsets, y, R, E, Kd, N, max_recv, elem_type,
-                          (hipStream_t)stream_, true);
-}
+#include "expert_gemm_entry.inc"
 
 const char* moe_a2a_route_plan(int T, int K) {
   if (T < 0 || K < 1) return "unknown";
