@@ -88,7 +88,9 @@ def parse_args():
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--workload", default="dsv3_rank")
-    p.add_argument("--combine", choices=["strict", "f32"], default="strict")
+    p.add_argument("--combine", choices=["strict", "f32"], default=None,
+                   help="default: what the workload's configuration names -- f32 accumulation for fp8_dispatch, the "
+                        "reference's rounding after every step (bit-identical) for the others")
     p.add_argument("--no-graph", action="store_true", help="launch eagerly from Python instead of a hipGraph")
     p.add_argument("--no-fuse-route", action="store_true", help="separate routing kernel even for small worlds")
     p.add_argument("--no-fuse-stub", action="store_true",
@@ -397,6 +399,8 @@ def main():
     cfg, W = wl.cfg, wl.world_size
     T, K, H, E = wl.total_tokens, cfg.experts_per_token, cfg.hidden_dim, cfg.num_experts
     fp8 = wl.fp8_dispatch and not args.bf16_dispatch
+    if args.combine is None:
+        args.combine = "f32" if fp8 else "strict"
     mode = contract.COMBINE_STRICT if args.combine == "strict" else contract.COMBINE_F32
     fuse_route, fuse_stub = not args.no_fuse_route, not args.no_fuse_stub
     tensors = concat_world(wl.world, dev)
@@ -511,8 +515,10 @@ def main():
             legs.insert(0, ("two_launches", mode, True))
         if mode == contract.COMBINE_STRICT:
             legs.append(("f32_combine", contract.COMBINE_F32, fuse_stub))
+        else:
+            legs.append(("strict_combine", contract.COMBINE_STRICT, fuse_stub))
         for name, leg_mode, leg_fuse in legs:
-            lib.moe_a2a_set_option(_lib.OPT_TWO_LAUNCHES, 0 if name == "f32_combine" else 1)
+            lib.moe_a2a_set_option(_lib.OPT_TWO_LAUNCHES, 0 if name in ("f32_combine", "strict_combine") else 1)
             other = Leg(torch, lib, wl, tensors, main, leg_mode, fp8, fuse_route, leg_fuse)
             o_ms = other.loop_wall(args.steps, args.warmup)
             o_per, _ = other.kernels(args.steps, args.warmup, o_ms * 1e3)
