@@ -71,6 +71,13 @@ class ForwardArgs(C.Structure):
 
 PROTOTYPES["moe_a2a_forward_packed"] = (_int, [C.POINTER(ForwardArgs)])
 
+# include/gemm_rs.h (same library)
+GEMM_RS_PROTOTYPES = {
+    "gemm_rs_workspace_bytes": (C.c_size_t, [_int, _int, _int, _int]),
+    "gemm_rs_forward": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _int, C.c_longlong, C.c_longlong, _int, _vp,
+                               C.c_size_t, _vp]),
+}
+
 _lib = None
 
 
@@ -90,7 +97,7 @@ def load() -> C.CDLL:
         raise RuntimeError(
             f"{LIB_PATH} is missing: build it with `python -m kernel_amd.build` (there is no fallback path)")
     lib = C.CDLL(LIB_PATH)
-    for name, (res, args) in PROTOTYPES.items():
+    for name, (res, args) in list(PROTOTYPES.items()) + list(GEMM_RS_PROTOTYPES.items()):
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

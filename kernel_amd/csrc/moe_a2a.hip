@@ -19,6 +19,8 @@
 //   dispatch_fold      dispatch, stub and weighted sum of a token behind a routing of its own
 //   expert_gemm        y[rows of e] = x[rows of e] * W_e^T, 128 x 128 tiles (short segments)
 //   expert_gemm_wide   the same on 256 x 256 tiles, software-pipelined; 16-bit or fp8 rows
+//   gemm_rs_*          the reference's other problem on one GPU: a K-split linear layer whose
+//                      reduce-scatter is the sum over the K shards held in one buffer
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <stdint.h>
@@ -27,6 +29,7 @@
 #include <algorithm>
 #include <atomic>
 
+#include "gemm_rs.h"
 #include "moe_a2a.h"
 
 // Scratch of moe_a2a_route_noalloc: the (tile, expert) count matrix of the multi-launch routing, held
@@ -74,12 +77,16 @@ enum KernelId {
   KID_FORWARD_TOKEN,
   KID_FORWARD_TILE,
   KID_DISPATCH_FOLD,
+  KID_GEMM_RS_WIDE,
+  KID_GEMM_RS_TILE,
+  KID_GEMM_RS_REDUCE,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
-    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token", "forward_tile", "dispatch_fold"};
+    "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token", "forward_tile", "dispatch_fold",
+    "gemm_rs_wide", "gemm_rs_tile", "gemm_rs_reduce"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -145,6 +152,7 @@ __device__ __forceinline__ float stub_factor(int e, int stub_kind, int num_exper
 #include "route_kernels.inc"
 #include "row_kernels.inc"
 #include "expert_gemm_kernels.inc"
+#include "gemm_rs_kernels.inc"
 
 // ---------------------------------------------------------------------------------------
 // host side
@@ -1034,6 +1042,7 @@ int moe_a2a_forward_packed(const moe_a2a_forward_args* a) {
 }
 
 #include "expert_gemm_entry.inc"
+#include "gemm_rs_entry.inc"
 
 const char* moe_a2a_route_plan(int T, int K) {
   if (T < 0 || K < 1) return "unknown";
