@@ -115,6 +115,10 @@ def parse_args():
     p.add_argument("--pow2-scales", action="store_true",
                    help="with --expert-gemm --fp8-weights on an fp8 workload: power-of-two scales for rows and weights, "
                         "multiplied with the scales as the matrix instruction's block exponents")
+    p.add_argument("--gemm-rs", default="", metavar="M,N,K[,bias]",
+                   help="measure the GEMM + reduce-scatter of the reference's other problem instead (8 emulated ranks "
+                        "as K shards of one buffer), e.g. 8192,8192,29568 or 512,4096,12288,bias; `all` runs the six "
+                        "benchmark shapes of gemm_rs/task.yml, one JSON line each")
     p.add_argument("--expert-gemm", type=int, default=0, metavar="N",
                    help="measure the grouped expert GEMM (N output columns per expert) on the workload's "
                         "dispatched rows instead of the dispatch/combine path")
@@ -395,6 +399,8 @@ def main():
         if lib.moe_a2a_set_option(getattr(_lib, "OPT_" + name), int(val, 0)) < 0:
             raise SystemExit(f"unknown option {name}")
 
+    if args.gemm_rs:
+        return gemm_rs_leg(args, lib, torch, dev)
     wl = contract.generate_workload(args.workload)
     cfg, W = wl.cfg, wl.world_size
     T, K, H, E = wl.total_tokens, cfg.experts_per_token, cfg.hidden_dim, cfg.num_experts
@@ -745,6 +751,86 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
                                    sample=f"first {done} of {E} experts ({rows_done} rows), f32 matmul; "
                                           f"worst error {worst:.2f} of the tolerance")
     print(json.dumps(out))
+
+
+def gemm_rs_leg(args, lib, torch, dev):
+    """GEMM + reduce-scatter of gemm_rs/reference.py:36-60 for a world of 8 ranks held as K shards of
+    one buffer.  One JSON line per shape: TFLOP/s of the whole world's product (2 M N K) against the
+    dense 16-bit MFMA peak, or GB/s when moving the operands once takes longer than the flops; the
+    reference's speed-of-light figure for the shape (task.yml:49-54: per GPU of an 8-GPU node, so one
+    GPU doing all eight shares has eight times the flops to do); a CPU leg on sampled rows."""
+    from kernel_amd import gemm_rs as G
+
+    sol_us = {(64, 7168, 18432): 6.46, (512, 4096, 12288): 8.19, (2048, 2880, 2880): 23.04,
+              (4096, 4096, 4096): 65.54, (8192, 4096, 14336): 131.07, (8192, 8192, 29568): 379.43}
+    if args.gemm_rs == "all":
+        specs = G.BENCHMARK_SPECS
+    else:
+        parts = args.gemm_rs.split(",")
+        specs = [dict(world_size=8, m=int(parts[0]), n=int(parts[1]), k=int(parts[2]),
+                      has_bias=len(parts) > 3 and parts[3] == "bias", seed=1234)]
+    main = torch.cuda.Stream()
+    main.wait_stream(torch.cuda.current_stream())
+    for spec in specs:
+        W, m, n, k = spec["world_size"], spec["m"], spec["n"], spec["k"]
+        datas = [G.generate_input(r, **spec) for r in range(W)]
+        x, w, bias = G.pack_world(datas, dev)
+        op = G.HipGemmReduceScatter(W)
+        out = torch.empty((m, n), dtype=x.dtype, device=dev)
+        with torch.cuda.stream(main):
+            for _ in range(max(args.warmup, 2)):
+                op.forward(x, w, bias, out=out)
+            main.synchronize()
+            per = kernel_times(lib, lambda cnt: [op.forward(x, w, bias, out=out) for _ in range(cnt)], args.steps, torch)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(main)
+            for _ in range(args.steps):
+                op.forward(x, w, bias, out=out)
+            e1.record(main)
+            main.synchronize()
+        ms_step = e0.elapsed_time(e1) / args.steps
+        t_us = sum(statistics.fmean(v) for v in per.values())  # one or two kernels per call
+        kernel = max(per, key=lambda kk: statistics.fmean(per[kk]))
+        flops = 2.0 * m * n * k
+        tflops = flops / t_us / 1e6
+        ws = int(lib.gemm_rs_workspace_bytes(m, n, k, W))
+        line = dict(metric=f"GEMM + reduce-scatter TFLOP/s, 8 K-shards on one GPU, m{m} n{n} k{k}", value=round(tflops, 1),
+                    unit="TFLOP/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 5),
+                    higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
+                    config=dict(workload="gemm_rs", m=m, n=n, k=k, emulated_ranks=W, has_bias=spec["has_bias"],
+                                kernel=kernel, partial_products_workspace_bytes=ws),
+                    kernels_us=summarise(per), kernel_us=round(t_us, 2),
+                    reference_speed_of_light_us_per_gpu_of_8=sol_us.get((m, n, k)))
+        # operands cross HBM once; partial products of the split form are written and read once more
+        gemm_bytes = (m + n) * k * 2 + m * n * 2 + 2 * ws
+        if gemm_bytes / (HBM_PEAK_GBPS * 1e3) > flops / (MFMA_PEAK_TFLOPS * 1e6):
+            gbps = gemm_bytes / t_us / 1e3
+            line["roofline"] = dict(bound="hbm", achieved=round(gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
+                                    frac=round(gbps / HBM_PEAK_GBPS, 4), traffic=None)
+        else:
+            line["roofline"] = dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                                    frac=round(tflops / MFMA_PEAK_TFLOPS, 4), traffic=None)
+        if not args.no_cpu:
+            from oracle import gemm_rs as O  # checker and baseline only
+
+            rows = min(m, 64)
+            sample = [(d[0][:rows], d[1], d[2]) for d in datas]
+            t0, reps = time.perf_counter(), 0
+            while True:
+                want = O.ref_world(sample)
+                reps += 1
+                if time.perf_counter() - t0 > min(args.cpu_seconds, 10.0) or reps >= 20:
+                    break
+            dt = (time.perf_counter() - t0) / reps
+            ok, msg = O.check_implementation(want, out[:rows].cpu())
+            if not ok:
+                raise RuntimeError("GEMM + reduce-scatter outside the reference's tolerance on the sampled rows")
+            line["cpu_baseline"] = dict(value=round(2.0 * rows * n * k / dt / 1e12, 4), unit="TFLOP/s",
+                                        cores=torch.get_num_threads(), kind="port",
+                                        sample=f"first {rows} of {m} rows, every rank's bf16 matmul + bias and the sum "
+                                               f"over the ranks; the GPU rows are within the reference's tolerance")
+        print(json.dumps(line), flush=True)
+        del x, w, bias, out, datas
 
 
 def cpu_baseline(wl, mode, fp8, y_gpu, b_dc, budget_s):

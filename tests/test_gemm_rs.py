@@ -207,11 +207,14 @@ def test_reference_shapes_at_full_size(gpu_device, spec):
 @pytest.mark.gpu
 @pytest.mark.parametrize("form", [256, 128, 32])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-def test_each_kernel_form(gpu_device, options, form, dtype):
+@pytest.mark.parametrize("k", [1024, 1440, 4 * 72], ids=["k256", "k360", "k72"])
+def test_each_kernel_form(gpu_device, options, form, dtype, k):
     """256 x 256 tiles, 128 x 128 tiles and per-shard partial products on one shape with ragged
-    edges (M and N not multiples of the tiles)."""
+    edges (M and N not multiples of the tiles); local K a multiple of the 64-column slab, five slabs
+    and a short one (360: the wide tiles start the last slab of a shard early and mask what it
+    shares with the one before), and one slab and a bit (72)."""
     options.set("GEMM_TILE", form)
-    W, m, n, k = 4, 392, 600, 1024
+    W, m, n = 4, 392, 600
     g = torch.Generator().manual_seed(form)
     datas = [(((torch.rand((m, k // W), generator=g) * 2 - 1) * 0.05).to(dtype),
               ((torch.rand((n, k // W), generator=g) * 2 - 1) * 0.05).to(dtype),
