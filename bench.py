@@ -484,7 +484,7 @@ def main():
     roofline = dict(bound="hbm", kernel=dom_name, achieved=round(dom_bytes / dom_us / 1e3, 1), peak=HBM_PEAK_GBPS,
                     unit="GB/s", frac=round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBPS, 4),
                     bytes_per_launch=dom_bytes, avg_us=round(dom_us, 3),
-                    avg_us_is="launch-to-launch period in the hipGraph: the kernel's own duration from its HIP "
+                    avg_us_is="launch-to-launch period of back-to-back launches: the kernel's own duration from its HIP "
                               "events plus its share of the launch overhead (what a profiler's kernel trace "
                               "reports for back-to-back launches)",
                     kernel_only_us=round(dom_kernel_us, 3), traffic=traffic, traffic_source=traffic_source)

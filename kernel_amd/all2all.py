@@ -75,7 +75,10 @@ class Dispatched:
     meta: torch.Tensor  # [R,5] int32: e, source rank, token in rank, k, 0
     disp_x: torch.Tensor  # [R,H] in_dtype, or uint8 e4m3fn bits for fp8 dispatch
     disp_scale: Optional[torch.Tensor] = None  # [R,H/128] f32 (fp8 only)
-    status: Optional[torch.Tensor] = None  # [1] int32: 1 expert id out of range, 2 padded segment overflow
+    # [1] int32, bits: 1 an expert id was out of range, 2 a padded segment overflowed.  The kernels only
+    # ever set bits: the word belongs to the buffer set and keeps what earlier calls on it raised
+    # until the owner clears it (``status.zero_()``)
+    status: Optional[torch.Tensor] = None
     max_recv: int = 0  # > 0: padded layout, expert e owns rows [e*max_recv, (e+1)*max_recv)
 
     @property
