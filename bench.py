@@ -541,6 +541,10 @@ def main():
             del other
         lib.moe_a2a_set_option(_lib.OPT_TWO_LAUNCHES, 0)
 
+    # a profiler's interception slows the host's launches; wall clocks taken with one attached are
+    # not those of the path (its kernel trace is the thing to read then)
+    out["profiler_attached"] = any(k.startswith(("ROCPROF", "ROCP_", "ROCTRACER")) for k in os.environ) or \
+        "rocprofiler" in os.environ.get("LD_PRELOAD", "")
     if args.cold:
         # cold caches: overwrite 1 GiB (4x the 256 MB Infinity Cache) before every step
         flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
