@@ -380,7 +380,8 @@ static int route_impl(const int32_t* indices, const int32_t* rank_start, int src
   const size_t lds_w = (size_t)kRouteWaves * E * sizeof(int);
   const size_t lds_starts = (size_t)(W + 1) * sizeof(int);
   if (a.R <= kRouteTilesMaxRows) {
-    size_t lds = lds_w + 2 * (size_t)E * sizeof(int) + (kRouteWaves + 1) * sizeof(int) + lds_starts;
+    size_t lds = lds_w + (size_t)kRouteCopies * route_copy_stride(E) * sizeof(int) + (kRouteWaves + 1) * sizeof(int) +
+                 lds_starts;
     if (int rc = ensure_lds<route_tiles_kernel>(lds)) return rc;
     return launch(KID_ROUTE_TILES, route_tiles_kernel, dim3(ceil_div(a.R, kRouteThreads)), dim3(kRouteThreads), lds,
                   stream, a);
