@@ -437,7 +437,7 @@ def main():
                   else "routing+dispatch, stub kernel, combine")
 
     # the configuration custom_kernel runs (kernel_amd/submission.py): the expert stand-in folded
-    # into the combine, two launches per step at the default workload
+    # in: one launch per step at the default workload
     leg = Leg(torch, lib, wl, tensors, main, mode, fp8, fuse_route, fuse_stub)
     graph_ms_per_step = leg.graph_wall(args.steps, args.warmup, use_graph)
     # the headline wall clock: the same K steps as plain launches from a C loop (no graph boundary in

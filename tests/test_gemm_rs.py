@@ -243,3 +243,30 @@ def test_local_k_with_a_short_last_slab_and_one_rank(gpu_device):
         out = G.HipGemmReduceScatter(W).forward(x, w, b).cpu()
         ok, worst = within_one_rounding(out, O.exact_world(datas))
         assert ok, worst
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("form", [256, 128, 32])
+def test_shards_with_gaps_between_them(gpu_device, options, form):
+    """Shard strides of the C ABI: the shards of each operand lie further apart than their size."""
+    options.set("GEMM_TILE", form)
+    lib = _lib.load()
+    W, m, n, kl, gap_a, gap_b = 4, 264, 272, 128, 64, 200
+    g = torch.Generator().manual_seed(31)
+    datas = [(((torch.rand((m, kl), generator=g) * 2 - 1) * 0.05).to(torch.bfloat16),
+              ((torch.rand((n, kl), generator=g) * 2 - 1) * 0.05).to(torch.bfloat16), None) for _ in range(W)]
+    sa, sb = m * kl + gap_a, n * kl + gap_b
+    a = torch.full((W * sa,), float("nan"), dtype=torch.bfloat16, device=gpu_device)  # the gaps hold NaN
+    b = torch.full((W * sb,), float("nan"), dtype=torch.bfloat16, device=gpu_device)
+    for s, (x, w, _) in enumerate(datas):
+        a[s * sa:s * sa + m * kl] = x.to(gpu_device).reshape(-1)
+        b[s * sb:s * sb + n * kl] = w.to(gpu_device).reshape(-1)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=gpu_device)
+    need = int(lib.gemm_rs_workspace_bytes(m, n, kl * W, W))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=gpu_device)
+    rc = lib.gemm_rs_forward(a.data_ptr(), b.data_ptr(), None, out.data_ptr(), m, n, kl * W, W, sa, sb, _lib.BF16,
+                             ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ok, worst = within_one_rounding(out.cpu(), O.exact_world(datas))
+    assert ok, worst
