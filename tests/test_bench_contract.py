@@ -87,3 +87,24 @@ def test_traffic_record_counts_only_for_the_sources_it_was_measured_on(tmp_path)
     if os.path.exists(bench.TRAFFIC_FILE):
         for e in json.load(open(bench.TRAFFIC_FILE))["entries"]:
             assert {"workload", "kernel", "bytes", "source_hash", "commit", "fetch_kib", "write_kib"} <= set(e)
+
+
+@pytest.mark.gpu
+def test_gemm_rs_leg_prints_one_line_per_shape_with_its_roofline(gpu_device):
+    p = subprocess.run([sys.executable, BENCH, "--gemm-rs", "512,4096,12288,bias", "--steps", "5", "--warmup", "1",
+                        "--cpu-seconds", "1"], capture_output=True, text=True, cwd=ROOT, timeout=110)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [ln for ln in p.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1, lines
+    d = json.loads(lines[0])
+    assert d["unit"] == "TFLOP/s" and d["n_gpus"] == 1 and d["dtype"] == "bf16" and d["data"] == "synthetic"
+    c = d["config"]
+    assert c["workload"] == "gemm_rs" and (c["m"], c["n"], c["k"]) == (512, 4096, 12288) and c["emulated_ranks"] == 8
+    assert c["has_bias"] is True and "model" not in c
+    r = d["roofline"]
+    assert r["bound"] in ("mfma", "hbm") and 0 < r["frac"] < 1 and abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
+    assert 0 < d["value"] < 2500.0  # below the dense bf16 peak
+    assert abs(d["value"] - 2.0 * 512 * 4096 * 12288 / d["kernel_us"] / 1e6) < 0.5
+    assert d["reference_speed_of_light_us_per_gpu_of_8"] == 8.19
+    cb = d["cpu_baseline"]
+    assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
