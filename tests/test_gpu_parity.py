@@ -591,3 +591,46 @@ def test_custom_kernel_contract(gpu_device):
         ok, msg = check_implementation(data, out)
         assert ok, msg
         assert torch.equal(bits(out.cpu()), bits(ref_kernel(data).cpu()))
+
+
+@pytest.mark.gpu
+def test_buffer_sets_alternate_and_old_token_counts_are_dropped(gpu_device):
+    """Two buffer sets per token count alternate (a result stays valid until the second-next call with
+    that count), both are allocated on the first call, and only the most recently used counts are kept."""
+    E, K, H = 16, 2, 64
+    cfg = C.MoEConfig(E, K, H, 64, torch.bfloat16, torch.bfloat16)
+    ata = HipAllToAll(cfg, 0, 1, fuse_stub=True)
+    g = torch.Generator().manual_seed(5)
+
+    def inputs(T):
+        idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+        world = [C.RankData(T, idx, torch.rand(T, K, generator=g), torch.randn(T, H, generator=g).to(torch.bfloat16))]
+        return world, concat_world(world, gpu_device)
+
+    worlds = {}
+    for T in range(1, ata.MAX_CACHED_SHAPES + 4):  # more token counts than the cache keeps
+        world, (x, idx, w, rs) = inputs(T)
+        y = ata.forward(x, idx, w, rs)
+        torch.cuda.synchronize()
+        want = V.run_world(cfg, world, stub_kind=ata.stub_kind)["y"]
+        assert torch.equal(bits(y.cpu()), bits(want)), T
+        worlds[T] = (world, x, idx, w, rs, y, want)
+    assert len(ata._bufs) == ata.MAX_CACHED_SHAPES
+    kept = [key[0] for key in ata._bufs]
+    assert kept == list(range(4, ata.MAX_CACHED_SHAPES + 4))  # the oldest counts went first
+    assert all(s is not None for ring in ata._bufs.values() for s in ring["sets"])  # both sets exist at once
+    # the result of a call survives the next call with the same count and is reused by the one after
+    T = kept[-1]
+    world, x, idx, w, rs, y1, want = worlds[T]
+    y2 = ata.forward(x, idx, w, rs)
+    assert y2.data_ptr() != y1.data_ptr()
+    torch.cuda.synchronize()
+    assert torch.equal(bits(y1.cpu()), bits(want)) and torch.equal(bits(y2.cpu()), bits(want))
+    y3 = ata.forward(x, idx, w, rs)
+    assert y3.data_ptr() == y1.data_ptr()
+    # a dropped count comes back with fresh buffers and the right answer
+    world, x, idx, w, rs, _, want = worlds[1]
+    y = ata.forward(x, idx, w, rs)
+    torch.cuda.synchronize()
+    assert torch.equal(bits(y.cpu()), bits(want))
+    assert len(ata._bufs) == ata.MAX_CACHED_SHAPES
