@@ -102,6 +102,10 @@ struct Bf16 {
     f32x2_t v = {a, b};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
   }
+  // a rounded to bf16 and left where the arithmetic goes on, in f32: the conversion of the pair
+  // (0, a) puts bf16(a) into the high half of the word over zeros, which IS that f32 -- one
+  // instruction per element where packing two and taking them apart again costs one and a half
+  static __device__ __forceinline__ float round(float a) { return __uint_as_float(pack(0.f, a)); }
 };
 
 struct F16 {
@@ -121,6 +125,10 @@ struct F16 {
     uint32_t l = __builtin_bit_cast(uint16_t, (_Float16)a);
     uint32_t h = __builtin_bit_cast(uint16_t, (_Float16)b);
     return l | (h << 16);
+  }
+  static __device__ __forceinline__ float round(float a) {
+    asm("" : "+v"(a));  // as in pack: keep the multiply or add that made a out of the conversion
+    return (float)(_Float16)a;
   }
 };
 
