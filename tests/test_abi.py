@@ -222,3 +222,25 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmoe_a2a.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.load()
+
+
+def test_headers_are_plain_c_and_link_from_c(tmp_path):
+    """The boundary is a C ABI: both headers compile as C99 with warnings on, and a C program links
+    against the library and calls an entry point that touches no GPU."""
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "abi.c"
+    src.write_text('#include "moe_a2a.h"\n#include "gemm_rs.h"\n'
+                   "int main(void) { moe_a2a_forward_args a; (void)a;\n"
+                   "  return (int)gemm_rs_workspace_bytes(0, 0, 0, 0) + moe_a2a_abi_version(); }\n")
+    inc = os.path.join(ROOT, "include")
+    lib_dir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I", inc, str(src)],
+                   check=True)
+    exe = tmp_path / "abi"
+    subprocess.run(["gcc", "-std=c99", "-I", inc, str(src), "-o", str(exe), "-L", lib_dir, "-lmoe_a2a",
+                    "-Wl,-rpath," + lib_dir], check=True)
+    assert subprocess.run([str(exe)]).returncode == _lib.ABI_VERSION

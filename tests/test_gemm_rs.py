@@ -270,3 +270,40 @@ def test_shards_with_gaps_between_them(gpu_device, options, form):
     torch.cuda.synchronize()
     ok, worst = within_one_rounding(out.cpu(), O.exact_world(datas))
     assert ok, worst
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(8, 64, 512, 8 * 256), (4, 520, 520, 4 * 128)], ids=["partial-products", "tiles"])
+def test_replays_of_a_captured_graph_follow_their_inputs(gpu_device, shape):
+    """The entry point only enqueues kernels (the grouped form: the tile kernel, then the reduction
+    over its partial products in the caller's workspace), so a call can be captured into a hipGraph;
+    every replay is checked against an eager run on the inputs of the moment, with eager work and
+    synchronisations between the replays."""
+    W, m, n, k = shape
+    op = G.HipGemmReduceScatter(W)
+    g = torch.Generator().manual_seed(77)
+    fresh = lambda: (((torch.rand((W, m, k // W), generator=g) * 2 - 1) * 0.05).to(torch.bfloat16).to(gpu_device),
+                     ((torch.rand((W, n, k // W), generator=g) * 2 - 1) * 0.05).to(torch.bfloat16).to(gpu_device),
+                     ((torch.rand((n,), generator=g) * 2 - 1) * 0.05).to(torch.bfloat16).to(gpu_device))
+    x, w, b = fresh()
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=gpu_device)
+    op.forward(x, w, b, out=out)  # allocates the workspace outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            op.forward(x, w, b, out=out)
+    for _ in range(3):
+        nx, nw, nb = fresh()
+        x.copy_(nx), w.copy_(nw), b.copy_(nb)
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = G.HipGemmReduceScatter(W).forward(x, w, b)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), eager.view(torch.int16))
+        ok, worst = within_one_rounding(got.cpu(), O.exact_world([(x[s].cpu(), w[s].cpu(), b.cpu()) for s in range(W)]))
+        assert ok, worst
