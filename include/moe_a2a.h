@@ -16,8 +16,9 @@
  *   - every pointer is a DEVICE pointer into caller-owned memory unless marked host;
  *   - the library allocates nothing, never synchronises, reads no environment variable and
  *     keeps no mutable state besides the opt-in launch timer and the option switches at the
- *     end of this file (both off unless the caller turns them on); every launch goes to the
- *     stream passed in, so a call sequence can be captured into a hipGraph;
+ *     end of this file (both off unless the caller turns them on: a launch then reads one atomic
+ *     flag and nothing else that is shared); every launch goes to the stream passed in, so a call
+ *     sequence can be captured into a hipGraph;
  *   - return value: 0 success, < 0 argument error found on the host before any
  *     launch (MOE_A2A_E_*), > 0 a hipError_t reported by the launch.
  */
@@ -31,7 +32,7 @@
 extern "C" {
 #endif
 
-#define MOE_A2A_ABI_VERSION 4
+#define MOE_A2A_ABI_VERSION 5
 
 /* element types of activations */
 #define MOE_A2A_F16 0
@@ -55,8 +56,10 @@ extern "C" {
 #define MOE_A2A_FP8_SCALE_F32 0
 #define MOE_A2A_FP8_SCALE_POW2 1
 
-/* bits of the status word the routing entry points write (OR-ed into what the word holds, so the
- * caller clears it; a call that meets both conditions reports both) */
+/* bits of the status word the routing entry points write (OR-ed into what the word holds: a call
+ * that meets both conditions reports both, and the word keeps what earlier calls raised until its
+ * owner clears it -- by a fill of its own, or without a launch through
+ * moe_a2a_forward_args.clear_status) */
 #define MOE_A2A_STATUS_BAD_EXPERT 1 /* an expert id was outside [0, E) and has been clamped      */
 #define MOE_A2A_STATUS_OVERFLOW 2   /* padded layout: an expert has more than max_recv entries   */
 
@@ -235,9 +238,9 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                     size_t workspace_bytes, moe_a2a_stream_t stream);
 
 /*
- * moe_a2a_forward with its arguments in a struct (same order, same meaning): a caller that repeats
- * the call fills the struct once and patches the pointers that change, which costs a foreign-function
- * binding one argument instead of thirty-one.
+ * moe_a2a_forward with its arguments in a struct (same order, same meaning, plus clear_status): a
+ * caller that repeats the call fills the struct once and patches the pointers that change, which
+ * costs a foreign-function binding one argument instead of thirty-one.
  */
 typedef struct moe_a2a_forward_args {
   const void* x;
@@ -254,6 +257,11 @@ typedef struct moe_a2a_forward_args {
   void* workspace;
   size_t workspace_bytes;
   moe_a2a_stream_t stream;
+  /* NULL, or one int32 that the first kernel of the call sets to 0.  A caller that alternates
+   * between two sets of buffers names the status word of the OTHER set here: the next call, which
+   * runs on that set behind this one on the stream, then starts from a cleared word and its status
+   * describes that call alone, with no launch spent on clearing.  Must not be this call's `status`. */
+  int32_t* clear_status;
 } moe_a2a_forward_args;
 int moe_a2a_forward_packed(const moe_a2a_forward_args* args);
 
@@ -338,9 +346,10 @@ int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w
                             moe_a2a_stream_t stream);
 
 /*
- * Launch timer (opt-in, process-wide, single caller thread).  Between begin and end every
- * kernel the library launches carries a pair of HIP events bound to that dispatch, so the
- * reported time is the kernel's own begin-to-end duration on the GPU.
+ * Launch timer (opt-in, process-wide).  Between begin and end every kernel the library launches,
+ * from any thread, carries a pair of HIP events bound to that dispatch, so the reported time is the
+ * kernel's own begin-to-end duration on the GPU; while the timer is on, launches are serialised on
+ * a mutex (a measurement aid: a product run leaves it off and pays one relaxed atomic read).
  *   begin(capacity)  allocate `capacity` event pairs and start recording
  *   end(ids, us, n)  wait for the recorded launches, write up to n (kernel id, microseconds)
  *                    pairs to HOST arrays, release the events; returns the number written
@@ -359,8 +368,12 @@ const char* moe_a2a_kernel_name(int kernel_id);
  * force one of several kernels that give the same results, for tests that compare the kernels with
  * each other and for measurements; they are plain integers read at launch time, so a caller that
  * never sets one pays nothing and sees no hidden behaviour.
- *   set_option(option, value)  returns the previous value, or MOE_A2A_E_DTYPE for an unknown option
+ *   set_option(option, value)  returns the previous value (>= 0), MOE_A2A_E_DTYPE for an unknown
+ *                              option or MOE_A2A_E_SHAPE for a negative value (no option takes one,
+ *                              so a negative return is always an error)
  *   get_option(option)         current value, or MOE_A2A_E_DTYPE
+ * A value is read when an entry point runs: a workspace size queried under one setting, or a
+ * hipGraph captured under it, belongs to that setting.
  */
 #define MOE_A2A_OPT_ROUTE_TILE 0    /* 1: moe_a2a_route_dispatch takes the token-tile kernel at any size   */
 #define MOE_A2A_OPT_GEMM_TILE 1     /* 32 | 128 | 256: tile family of the expert GEMM entry points          */

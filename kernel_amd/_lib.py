@@ -9,7 +9,7 @@ import os
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmoe_a2a.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 F16, BF16 = 0, 1
 FP8_SCALE_F32, FP8_SCALE_POW2 = 0, 1
 STATUS_BAD_EXPERT, STATUS_OVERFLOW = 1, 2  # bits of the routing status word
@@ -66,7 +66,7 @@ class ForwardArgs(C.Structure):
                                         "fp8_dispatch", "stub_kind", "combine_mode", "fuse_route", "fuse_stub")] +
                 [(n, C.c_void_p) for n in ("counts", "offsets", "slot_of_entry", "src_of_slot", "meta", "status", "disp",
                                            "disp_scale", "expert_y", "out", "workspace")] +
-                [("workspace_bytes", C.c_size_t), ("stream", C.c_void_p)])
+                [("workspace_bytes", C.c_size_t), ("stream", C.c_void_p), ("clear_status", C.c_void_p)])
 
 
 PROTOTYPES["moe_a2a_forward_packed"] = (_int, [C.POINTER(ForwardArgs)])

@@ -18,6 +18,7 @@ torch is used for device memory and the current stream only.
 from __future__ import annotations
 
 import collections
+import copy
 import ctypes
 import dataclasses
 from typing import Optional, Sequence
@@ -75,9 +76,10 @@ class Dispatched:
     meta: torch.Tensor  # [R,5] int32: e, source rank, token in rank, k, 0
     disp_x: torch.Tensor  # [R,H] in_dtype, or uint8 e4m3fn bits for fp8 dispatch
     disp_scale: Optional[torch.Tensor] = None  # [R,H/128] f32 (fp8 only)
-    # [1] int32, bits: 1 an expert id was out of range, 2 a padded segment overflowed.  The kernels only
-    # ever set bits: the word belongs to the buffer set and keeps what earlier calls on it raised
-    # until the owner clears it (``status.zero_()``)
+    # [1] int32, bits: 1 an expert id was out of range, 2 a padded segment overflowed.  It describes
+    # the call that produced this record and stays readable until the next call on the same
+    # ``HipAllToAll`` is enqueued (that call clears the word for the call after it: the host class
+    # alternates between two buffer sets, and each call clears the other set's word)
     status: Optional[torch.Tensor] = None
     max_recv: int = 0  # > 0: padded layout, expert e owns rows [e*max_recv, (e+1)*max_recv)
 
@@ -124,7 +126,9 @@ class HipAllToAll:
                  fuse_stub: bool = False, padded: bool = False, max_recv: Optional[int] = None):
         if cfg.num_experts % world_size:
             raise ValueError("num_experts must be a multiple of world_size")
-        self.cfg = cfg
+        # a copy: buffers and checks belong to the values the instance was built for, also when the
+        # caller changes its config object in place afterwards
+        self.cfg = cfg = copy.copy(cfg)
         self.rank = rank
         self.world_size = world_size
         self.num_local_experts = cfg.num_experts // world_size
@@ -169,6 +173,8 @@ class HipAllToAll:
         # does not meet an allocation either
         for i in (0, 1):
             ring["sets"][i] = self._allocate(T, device)
+        for i in (0, 1):  # a call on one set clears the status word of the other (see Dispatched.status)
+            ring["sets"][i]["partner_status"] = ring["sets"][i ^ 1]["status"]
         return ring["sets"][ring["cur"]]
 
     def _allocate(self, T: int, device) -> dict:
@@ -224,6 +230,7 @@ class HipAllToAll:
             if rank_start.dtype != torch.int32 or rank_start.numel() != W + 1:
                 raise ValueError("rank_start must be int32[world_size + 1]")
         b = self._buffers(T, dp_x.device, advance=True)
+        b["status"].zero_()  # the phase-by-phase entry points only ever set bits: the record describes this call
         lib, st = self.lib, _stream()
         pad = self.max_recv if self.padded else 0
         route_out = (_ptr(b["counts"]), _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]),
@@ -372,7 +379,7 @@ class HipAllToAll:
                 self.stub_kind, self.combine_mode, fuse_route, int(self.fuse_stub), _ptr(b["counts"]),
                 _ptr(b["offsets"]), _ptr(b["slot_of_entry"]), _ptr(b["src_of_slot"]), _ptr(b["meta"]),
                 _ptr(b["status"]), _ptr(b["disp_x"]), _ptr(b["disp_scale"]), _ptr(b["expert_y"]), _ptr(b["out"]),
-                _ptr(b["workspace"]), b["workspace"].numel(), stream)
+                _ptr(b["workspace"]), b["workspace"].numel(), stream, _ptr(b["partner_status"]))
 
     def _check_inputs(self, x, indices, weights, rank_start) -> None:
         cfg = self.cfg
@@ -397,10 +404,18 @@ class HipAllToAll:
                           self.max_recv if self.padded else 0)
 
     def forward(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
-                rank_start: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                rank_start: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                check_status: bool = False) -> torch.Tensor:
         """dispatch -> stub -> combine in one library call; returns ``y[T,H]``: ``out`` if given
         (``out_dtype[>=T,H]``, contiguous), else a buffer the second-next call reuses.
-        ``self.last`` holds the ``Dispatched`` record of the call."""
+        ``self.last`` holds the ``Dispatched`` record of the call.
+
+        ``check_status=True`` reads the call's status word back (this synchronises) and raises where
+        the reference would: ``IndexError`` for an expert id outside ``[0, num_experts)`` (the
+        reference indexes ``token_map[dst_rank]``, all2all/reference.py:81-86), ``RuntimeError`` for
+        a padded segment with more than ``max_recv`` rows (reference.py:140-146 would write past
+        ``expert_x[local_eid]``).  Without it such ids are clamped and the bits stay in
+        ``self.last.status`` until the next call."""
         cfg = self.cfg
         T = x.shape[0]
         if T == 0:
@@ -434,7 +449,22 @@ class HipAllToAll:
         if rc:
             raise _lib.MoeA2AError(rc, "moe_a2a_forward")
         self.last = b["_record"]
+        if check_status:
+            self.raise_on_status(b["status"])
         return b["out"] if out is None else out
+
+    @staticmethod
+    def raise_on_status(status: torch.Tensor) -> None:
+        """Read a status word back (synchronises); clear it and raise if a bit is set."""
+        bits = int(status.item())
+        if not bits:
+            return
+        status.zero_()
+        if bits & _lib.STATUS_BAD_EXPERT:
+            raise IndexError("an expert id lies outside [0, num_experts): the reference fails on it at "
+                             "token_map[dst_rank] (all2all/reference.py:81-86); the kernels clamped it")
+        raise RuntimeError("a padded expert segment holds more than max_recv rows (status bit "
+                           f"{_lib.STATUS_OVERFLOW}): the extra entries were folded onto its last row")
 
     def plan(self, x: torch.Tensor, indices: torch.Tensor, weights: torch.Tensor,
              rank_start: Optional[torch.Tensor] = None, stream: Optional[torch.cuda.Stream] = None):

@@ -28,6 +28,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 
 #include "gemm_rs.h"
 #include "moe_a2a.h"
@@ -175,6 +176,11 @@ struct LaunchTimer {
   int* ids = nullptr;
 };
 LaunchTimer g_timer;
+// A launch looks at this flag only (relaxed: the timer is off in a product run and the launch path
+// then touches no shared mutable state); while it is set, launches, begin, skip and end take the
+// mutex, so a second caller thread's launches are recorded one at a time instead of racing.
+std::atomic<bool> g_timer_on{false};
+std::mutex g_timer_mutex;
 
 template <typename T>
 struct same_type {
@@ -185,6 +191,11 @@ struct same_type {
 template <typename... KArgs>
 int launch(int kid, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t stream,
            typename same_type<KArgs>::type... args) {
+  if (!g_timer_on.load(std::memory_order_relaxed)) {
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
+    return (int)hipGetLastError();
+  }
+  std::lock_guard<std::mutex> hold(g_timer_mutex);
   if (g_timer.active && g_timer.skip > 0) {
     --g_timer.skip;
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
@@ -373,7 +384,7 @@ static int static_scratch(int32_t** out) {
 static int route_impl(const int32_t* indices, const int32_t* rank_start, int src_rank, int T, int K, int E, int W,
                       int max_recv, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot,
                       int32_t* meta, int32_t* status, void* workspace, size_t workspace_bytes, bool static_ok,
-                      moe_a2a_stream_t stream_) {
+                      moe_a2a_stream_t stream_, int32_t* clear_status = nullptr) {
   if (int rc = check_route_shape(T, K, E, W)) return rc;
   if (max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
   if (!counts || !offsets) return MOE_A2A_E_NULL;
@@ -382,9 +393,10 @@ static int route_impl(const int32_t* indices, const int32_t* rank_start, int src
   // No token: counts and offsets are zero and nothing else is written.  A kernel of its own, which
   // is never handed `indices` (NULL is allowed here), does that.
   if (T == 0)
-    return launch(KID_ROUTE_EMPTY, route_empty_kernel, dim3(1), dim3(kRouteThreads), 0, stream, counts, offsets, E);
+    return launch(KID_ROUTE_EMPTY, route_empty_kernel, dim3(1), dim3(kRouteThreads), 0, stream, counts, offsets, E,
+                  clear_status);
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
-              slot_of_entry, src_of_slot, meta, status};
+              slot_of_entry, src_of_slot, meta, status, clear_status};
   const size_t lds_w = (size_t)kRouteWaves * E * sizeof(int);
   const size_t lds_starts = (size_t)(W + 1) * sizeof(int);
   if (a.R <= kRouteTilesMaxRows) {
@@ -509,21 +521,21 @@ int moe_a2a_fused_ok(int T, int K, int H) {
   return (long long)tile_tokens(T, K, H) * H >= 2ll * T ? 1 : 0;
 }
 
-int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
-                           int K, int E, int W, int H, int max_recv, int32_t* counts, int32_t* offsets,
-                           int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
-                           void* disp_x, moe_a2a_stream_t stream_) {
+static int route_dispatch_impl(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
+                               int K, int E, int W, int H, int max_recv, int32_t* counts, int32_t* offsets,
+                               int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
+                               void* disp_x, moe_a2a_stream_t stream_, int32_t* clear_status) {
   if (int rc = check_route_shape(T, K, E, W)) return rc;
   if (max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
   if (int rc = check_rows(x, disp_x, T, K, H, 8)) return rc;
   if (!counts || !offsets) return MOE_A2A_E_NULL;
   if (T > 0 && (!indices || !slot_of_entry || !src_of_slot || !meta)) return MOE_A2A_E_NULL;
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
-              slot_of_entry, src_of_slot, meta, status};
+              slot_of_entry, src_of_slot, meta, status, clear_status};
   const int nvec = H / 8;
   if (!fused_small_ok(T, K, H) || option(MOE_A2A_OPT_ROUTE_TILE) == 1) {  // token tiles: any table size
-    if (T == 0) return moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets,
-                                     slot_of_entry, src_of_slot, meta, status, nullptr, 0, stream_);
+    if (T == 0) return route_impl(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
+                                  src_of_slot, meta, status, nullptr, 0, false, stream_, clear_status);
     if (K > kTileMaxOwn) return MOE_A2A_E_SHAPE;
     const int tile = tile_tokens(T, K, H);
     dim3 grid((unsigned)ceil_div(T, tile)), block(kTileThreads);
@@ -557,6 +569,14 @@ int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t*
   CALL_FUSED(32);
 #undef CALL_FUSED3
 #undef CALL_FUSED
+}
+
+int moe_a2a_route_dispatch(const void* x, const int32_t* indices, const int32_t* rank_start, int src_rank, int T,
+                           int K, int E, int W, int H, int max_recv, int32_t* counts, int32_t* offsets,
+                           int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta, int32_t* status,
+                           void* disp_x, moe_a2a_stream_t stream) {
+  return route_dispatch_impl(x, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts, offsets, slot_of_entry,
+                             src_of_slot, meta, status, disp_x, stream, nullptr);
 }
 
 int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry, uint8_t* disp_q,
@@ -916,14 +936,14 @@ static int forward_one_launch(const void* x, const int32_t* indices, const float
                               int src_rank, int T, int K, int E, int W, int H, int elem_type, int stub_kind,
                               int combine_mode, int32_t* counts, int32_t* offsets, int32_t* slot_of_entry,
                               int32_t* src_of_slot, int32_t* meta, int32_t* status, void* disp, void* out,
-                              hipStream_t stream) {
+                              hipStream_t stream, int32_t* clear_status) {
   if (int rc = check_route_shape(T, K, E, W)) return rc;
   if (int rc = check_rows(x, disp, T, K, H, 8)) return rc;
   if (!aligned16(out)) return MOE_A2A_E_ALIGN;
   if (!counts || !offsets || !indices || !weights || !slot_of_entry || !src_of_slot || !meta || !out)
     return MOE_A2A_E_NULL;
   RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), 0, counts, offsets,
-              slot_of_entry, src_of_slot, meta, status};
+              slot_of_entry, src_of_slot, meta, status, clear_status};
   const int nvec = H / 8;
   const int E_l = E / W;
   if (forward_one_launch_form(T, K, H, 0, elem_type, elem_type, 0) == 2) {
@@ -985,12 +1005,12 @@ static int forward_one_launch(const void* x, const int32_t* indices, const float
 #undef FWD_ARGS
 }
 
-int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
-                    int src_rank, int T, int K, int E, int W, int H, int max_recv, int in_type, int out_type,
-                    int fp8_dispatch, int stub_kind, int combine_mode, int fuse_route, int fuse_stub,
-                    int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
-                    int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
-                    size_t workspace_bytes, moe_a2a_stream_t stream) {
+static int forward_impl(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
+                        int src_rank, int T, int K, int E, int W, int H, int max_recv, int in_type, int out_type,
+                        int fp8_dispatch, int stub_kind, int combine_mode, int fuse_route, int fuse_stub,
+                        int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
+                        int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
+                        size_t workspace_bytes, moe_a2a_stream_t stream, int32_t* clear_status) {
   if (!known_type(in_type) || !known_type(out_type)) return MOE_A2A_E_DTYPE;
   if (fp8_dispatch < 0 || fp8_dispatch > 2) return MOE_A2A_E_DTYPE;
   if (fp8_dispatch && !disp_scale) return MOE_A2A_E_NULL;
@@ -1001,10 +1021,10 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
       forward_one_launch_ok(T, K, H, max_recv, in_type, out_type, fp8_dispatch))
     return forward_one_launch(x, indices, weights, rank_start, src_rank, T, K, E, W, H, in_type, stub_kind,
                               combine_mode, counts, offsets, slot_of_entry, src_of_slot, meta, status, disp, out,
-                              (hipStream_t)stream);
+                              (hipStream_t)stream, clear_status);
   if (T > 0 && fuse_stub && dispatch_fold_ok(T, K, H, max_recv, in_type, out_type, fp8_dispatch, fuse_route)) {
-    if (int rc = moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
-                               src_of_slot, meta, status, workspace, workspace_bytes, stream))
+    if (int rc = route_impl(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
+                            src_of_slot, meta, status, workspace, workspace_bytes, false, stream, clear_status))
       return rc;
     if (fp8_dispatch)
       return dispatch_fold_fp8(x, indices, weights, slot_of_entry, disp, disp_scale, out, T, K, E, W, H, in_type,
@@ -1015,12 +1035,12 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
   const bool fused = !fp8_dispatch && T > 0 &&
                      (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
   if (fused) {
-    if (int rc = moe_a2a_route_dispatch(x, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts, offsets,
-                                        slot_of_entry, src_of_slot, meta, status, disp, stream))
+    if (int rc = route_dispatch_impl(x, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts, offsets,
+                                     slot_of_entry, src_of_slot, meta, status, disp, stream, clear_status))
       return rc;
   } else {
-    if (int rc = moe_a2a_route(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
-                               src_of_slot, meta, status, workspace, workspace_bytes, stream))
+    if (int rc = route_impl(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,
+                            src_of_slot, meta, status, workspace, workspace_bytes, false, stream, clear_status))
       return rc;
     if (int rc = fp8_dispatch ? moe_a2a_dispatch_fp8(x, in_type, slot_of_entry, (uint8_t*)disp, disp_scale, T, K, H,
                                                      fp8_dispatch == 2 ? MOE_A2A_FP8_SCALE_POW2
@@ -1041,13 +1061,25 @@ int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights,
                       (long long)T * K * H * (fp8_dispatch ? 1 : 2), stream);
 }
 
+int moe_a2a_forward(const void* x, const int32_t* indices, const float* weights, const int32_t* rank_start,
+                    int src_rank, int T, int K, int E, int W, int H, int max_recv, int in_type, int out_type,
+                    int fp8_dispatch, int stub_kind, int combine_mode, int fuse_route, int fuse_stub,
+                    int32_t* counts, int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
+                    int32_t* status, void* disp, float* disp_scale, void* expert_y, void* out, void* workspace,
+                    size_t workspace_bytes, moe_a2a_stream_t stream) {
+  return forward_impl(x, indices, weights, rank_start, src_rank, T, K, E, W, H, max_recv, in_type, out_type,
+                      fp8_dispatch, stub_kind, combine_mode, fuse_route, fuse_stub, counts, offsets, slot_of_entry,
+                      src_of_slot, meta, status, disp, disp_scale, expert_y, out, workspace, workspace_bytes, stream,
+                      nullptr);
+}
+
 int moe_a2a_forward_packed(const moe_a2a_forward_args* a) {
   if (!a) return MOE_A2A_E_NULL;
-  return moe_a2a_forward(a->x, a->indices, a->weights, a->rank_start, a->src_rank, a->T, a->K, a->E, a->W, a->H,
+  return forward_impl(a->x, a->indices, a->weights, a->rank_start, a->src_rank, a->T, a->K, a->E, a->W, a->H,
                          a->max_recv, a->in_type, a->out_type, a->fp8_dispatch, a->stub_kind, a->combine_mode,
                          a->fuse_route, a->fuse_stub, a->counts, a->offsets, a->slot_of_entry, a->src_of_slot, a->meta,
-                         a->status, a->disp, a->disp_scale, a->expert_y, a->out, a->workspace, a->workspace_bytes,
-                         a->stream);
+                      a->status, a->disp, a->disp_scale, a->expert_y, a->out, a->workspace, a->workspace_bytes,
+                      a->stream, a->clear_status);
 }
 
 #include "expert_gemm_entry.inc"
@@ -1060,6 +1092,7 @@ const char* moe_a2a_route_plan(int T, int K) {
 
 int moe_a2a_set_option(int which, int value) {
   if (which < 0 || which >= MOE_A2A_OPT_COUNT) return MOE_A2A_E_DTYPE;
+  if (value < 0) return MOE_A2A_E_SHAPE;  // no option takes a negative value, so a return below zero is always an error
   return g_option[which].exchange(value, std::memory_order_relaxed);
 }
 
@@ -1069,6 +1102,7 @@ int moe_a2a_get_option(int which) {
 }
 
 int moe_a2a_timer_begin(int capacity) {
+  std::lock_guard<std::mutex> hold(g_timer_mutex);
   if (g_timer.active || capacity < 1) return MOE_A2A_E_STATE;
   g_timer.start = new hipEvent_t[capacity];
   g_timer.stop = new hipEvent_t[capacity];
@@ -1094,18 +1128,22 @@ int moe_a2a_timer_begin(int capacity) {
   g_timer.used = 0;
   g_timer.skip = 0;
   g_timer.active = true;
+  g_timer_on.store(true, std::memory_order_release);
   return 0;
 }
 
 int moe_a2a_timer_skip(int launches) {
+  std::lock_guard<std::mutex> hold(g_timer_mutex);
   if (!g_timer.active || launches < 0) return MOE_A2A_E_STATE;
   g_timer.skip = launches;
   return 0;
 }
 
 int moe_a2a_timer_end(int* kernel_ids, float* microseconds, int n) {
+  std::lock_guard<std::mutex> hold(g_timer_mutex);
   if (!g_timer.active) return MOE_A2A_E_STATE;
   g_timer.active = false;
+  g_timer_on.store(false, std::memory_order_release);
   int written = 0;
   for (int i = 0; i < g_timer.used; ++i) {
     (void)hipEventSynchronize(g_timer.stop[i]);

@@ -183,6 +183,9 @@ def test_option_switches(lib):
     assert lib.moe_a2a_set_option(_lib.OPT_GEMM_TILE, 0) == 128  # returns the previous value
     assert lib.moe_a2a_set_option(-1, 1) == E_DTYPE and lib.moe_a2a_set_option(8, 1) == E_DTYPE
     assert lib.moe_a2a_get_option(99) == E_DTYPE
+    # no option takes a negative value, so a negative return always means an error
+    assert lib.moe_a2a_set_option(_lib.OPT_GEMM_TILE, -3) == E_SHAPE
+    assert lib.moe_a2a_get_option(_lib.OPT_GEMM_TILE) == 0
 
 
 def test_library_reads_no_environment_variable():

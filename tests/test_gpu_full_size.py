@@ -49,16 +49,25 @@ def test_full_size_against_oracle(gpu_device, name):
     assert torch.equal(bits(y2.cpu()), bits(want["y"]))
     # the one-call forward knows what the dispatch wrote and may pick other cache policies for the
     # combine (write-through output stores beyond 256 MB of dispatched rows): same bits, both modes
+    # ... and with the stub folded in it is what custom_kernel and bench.py run (for fp8_dispatch in
+    # f32 mode: the streaming stub_combine over fp8 rows that the bench line of that workload times)
     x, idx, w, rs = concat_world(wl.world, gpu_device)
+    folded = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fp8_dispatch=wl.fp8_dispatch,
+                         fuse_stub=True)
+    want32 = None
     for mode in (C.COMBINE_STRICT, C.COMBINE_F32):
-        ata.combine_mode = mode
-        y3 = ata.forward(x, idx, w, rs)
-        torch.cuda.synchronize()
-        if mode == C.COMBINE_STRICT:
-            assert torch.equal(bits(y3.cpu()), bits(want["y"]))
-        else:
-            want32 = V.run_world(wl.cfg, wl.world, stub_kind=wl.stub_kind, fp8=wl.fp8_dispatch, combine_mode=mode)["y"]
-            assert torch.equal(bits(y3.cpu()), bits(want32))
+        for host in (ata, folded):
+            host.combine_mode = mode
+            y3 = host.forward(x, idx, w, rs)
+            torch.cuda.synchronize()
+            assert int(host.last.status.item()) == 0
+            if mode == C.COMBINE_STRICT:
+                assert torch.equal(bits(y3.cpu()), bits(want["y"]))
+            else:
+                if want32 is None:
+                    want32 = V.run_world(wl.cfg, wl.world, stub_kind=wl.stub_kind, fp8=wl.fp8_dispatch,
+                                         combine_mode=mode)["y"]
+                assert torch.equal(bits(y3.cpu()), bits(want32))
 
 
 def test_fp8_rows_within_stated_bound_at_full_size(gpu_device):

@@ -524,7 +524,7 @@ def test_unaligned_index_slices_and_out_of_range_ids(gpu_device):
 
 def test_status_reports_both_conditions(gpu_device):
     """A call that meets an expert id out of range AND a padded segment that overflows reports both
-    bits, whichever lane gets there first; the word is sticky until the caller clears it."""
+    bits, whichever lane gets there first; the record of a later call describes that call alone."""
     wl = C.generate_workload("skew_world")
     x, idx, w, rs = concat_world(wl.world, gpu_device)
     bad = idx.clone()
@@ -536,11 +536,68 @@ def test_status_reports_both_conditions(gpu_device):
         ata.forward(x, bad, w, rs)
         torch.cuda.synchronize()
         assert int(ata.last.status.item()) == _lib.STATUS_BAD_EXPERT | _lib.STATUS_OVERFLOW
-        ata.last.status.zero_()
-        ata.forward(x, idx, w, rs)  # the other buffer set, clean ids: only the overflow is left
-        ata.forward(x, idx, w, rs)  # the first set again, after the caller cleared its word
-        torch.cuda.synchronize()
-        assert int(ata.last.status.item()) == _lib.STATUS_OVERFLOW
+        for _ in range(3):  # clean ids on the other buffer set, then on the first one again: only the overflow
+            ata.forward(x, idx, w, rs)
+            torch.cuda.synchronize()
+            assert int(ata.last.status.item()) == _lib.STATUS_OVERFLOW
+
+
+@pytest.mark.parametrize("name,fp8,fuse_route", [("tiny", False, True), ("dsv3_rank", False, True),
+                                                 ("skew_world", False, True), ("skew_world", False, False),
+                                                 ("skew_world", True, True), ("prefill_graph", False, True)])
+def test_status_describes_the_call_that_produced_it(gpu_device, name, fp8, fuse_route):
+    """The status word belongs to a reused buffer set and the kernels only set bits in it: every call
+    clears the word of the OTHER set (no launch of its own), so a clean call after a bad one reads 0
+    whichever set it lands on, through every form of the one-call forward and through the
+    phase-by-phase dispatch; `check_status` raises as the reference does (reference.py:81-86)."""
+    wl = C.generate_workload(name, tokens_scale=1 / 8 if name == "prefill_graph" else 1.0)
+    x, idx, w, rs = concat_world(wl.world, gpu_device)
+    bad = idx.clone()
+    bad[0, 0] = wl.cfg.num_experts
+    ata = HipAllToAll(wl.cfg, 0, wl.world_size, stub_kind=wl.stub_kind, fp8_dispatch=fp8, fuse_route=fuse_route,
+                      fuse_stub=True)
+    want = ata.forward(x, idx, w, rs).clone()
+    seen = []
+    for ids in (bad, idx, idx, bad, bad, idx, idx):
+        y = ata.forward(x, ids, w, rs)
+        seen.append(int(ata.last.status.item()))
+        if ids is idx:
+            assert torch.equal(bits(y.cpu()), bits(want.cpu()))
+    assert seen == [1, 0, 0, 1, 1, 0, 0]
+    with pytest.raises(IndexError, match="expert id"):
+        ata.forward(x, bad, w, rs, check_status=True)
+    ata.forward(x, idx, w, rs, check_status=True)  # and the clean call behind it passes
+    ata.forward(x, idx, w, rs, check_status=True)
+    # phase by phase: the record of a dispatch describes that dispatch
+    for ids, bits_want in ((bad, 1), (idx, 0), (idx, 0)):
+        assert int(ata.dispatch(x, ids, rs).status.item()) == bits_want
+
+
+def test_custom_kernel_check_status_and_config_changed_in_place(gpu_device):
+    """`custom_kernel(data, check_status=True)` raises on an id the reference would fail on; a config
+    object changed in place between two calls gets the instance of its new values."""
+    from kernel_amd.submission import custom_kernel
+    from oracle.checker import ref_kernel
+
+    spec = dict(C.REFERENCE_TESTS[1])
+    W = spec.pop("world_size")
+    cfg, rd, rank, world = C.generate_input(**spec, rank=2, world_size=W, device=gpu_device)
+    out = custom_kernel((cfg, rd, rank, world), check_status=True)
+    assert torch.equal(bits(out.cpu()), bits(ref_kernel((cfg, rd, rank, world)).cpu()))
+    bad = C.RankData(rd.num_tokens, rd.indices.clone(), rd.weights, rd.x)
+    bad.indices[0, 0] = cfg.num_experts + 1
+    with pytest.raises(IndexError):
+        custom_kernel((cfg, bad, rank, world), check_status=True)
+    custom_kernel((cfg, bad, rank, world))  # default: clamped, no error
+    # same object, other geometry: half the hidden size and another top-k
+    T = rd.num_tokens
+    cfg.hidden_dim //= 2
+    cfg.experts_per_token -= 1
+    rd2 = C.RankData(T, rd.indices[:, :cfg.experts_per_token].contiguous(),
+                     rd.weights[:, :cfg.experts_per_token].contiguous(), rd.x[:, :cfg.hidden_dim].contiguous())
+    out2 = custom_kernel((cfg, rd2, rank, world), check_status=True)
+    assert out2.shape == (T, cfg.hidden_dim)
+    assert torch.equal(bits(out2.cpu()), bits(ref_kernel((cfg, rd2, rank, world)).cpu()))
 
 
 def test_dispatch_of_an_empty_rank(gpu_device):

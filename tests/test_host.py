@@ -88,3 +88,42 @@ def test_product_path_refuses_cpu_tensors():
 def test_constructor_checks_expert_split():
     with pytest.raises(ValueError):
         HipAllToAll(C.MoEConfig(10, 2, 64, 8), 0, 4)
+
+
+def test_custom_kernel_instance_follows_the_config_values(monkeypatch):
+    """The memo of `custom_kernel` is keyed by the config's VALUES, read at every call: a config
+    changed in place never meets an instance (and buffers) built for its old values, and the
+    instance keeps a copy of the config it was built for."""
+    from kernel_amd import submission as S
+
+    made = []
+
+    class Recorder:
+        def __init__(self, cfg, rank, world_size, **kw):
+            self.key = (cfg.num_experts, cfg.experts_per_token, cfg.hidden_dim)
+            made.append(self)
+
+    monkeypatch.setattr(S, "HipAllToAll", Recorder)
+    monkeypatch.setattr(S, "_instances", {})
+    monkeypatch.setattr(S, "_last", [None, None])
+    cfg = C.MoEConfig(64, 6, 2048, 32)
+    a = S._instance(cfg, 0, 8, "cuda:0", 0, 0)
+    assert S._instance(cfg, 0, 8, "cuda:0", 0, 0) is a and len(made) == 1
+    cfg.hidden_dim = 4096  # in place
+    b = S._instance(cfg, 0, 8, "cuda:0", 0, 0)
+    assert b is not a and b.key == (64, 6, 4096)
+    cfg.experts_per_token = 4
+    c = S._instance(cfg, 0, 8, "cuda:0", 0, 0)
+    assert c is not a and c is not b and c.key == (64, 4, 4096)
+    cfg.hidden_dim, cfg.experts_per_token = 2048, 6  # back to the first values: the first instance again
+    assert S._instance(cfg, 0, 8, "cuda:0", 0, 0) is a and len(made) == 3
+    other = C.MoEConfig(64, 6, 2048, 32)  # an equal config in another object shares it
+    assert S._instance(other, 0, 8, "cuda:0", 0, 0) is a
+    assert S._instance(other, 1, 8, "cuda:0", 0, 0) is not a  # another rank does not
+
+
+def test_host_object_keeps_its_own_copy_of_the_config():
+    cfg = C.MoEConfig(64, 6, 2048, 32)
+    ata = HipAllToAll(cfg, 0, 8)
+    cfg.hidden_dim = 64
+    assert ata.cfg.hidden_dim == 2048 and ata.cfg is not cfg
