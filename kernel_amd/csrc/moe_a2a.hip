@@ -161,6 +161,7 @@ __device__ __forceinline__ float stub_factor(int e, int stub_kind, int num_exper
 #include "route_kernels.inc"
 #include "row_kernels.inc"
 #include "expert_gemm_kernels.inc"
+#include "gemm8_kernels.inc"
 #include "gemm_rs_kernels.inc"
 
 // ---------------------------------------------------------------------------------------

@@ -31,14 +31,30 @@ def test_without_a_gpu_the_bench_fails_instead_of_measuring_the_cpu():
 @pytest.mark.gpu
 def test_json_line_has_the_contract_keys(gpu_device):
     p = subprocess.run([sys.executable, BENCH, "--steps", "20", "--warmup", "4", "--cpu-seconds", "1"],
-                       capture_output=True, text=True, cwd=ROOT, timeout=110)
+                       capture_output=True, text=True, cwd=ROOT, timeout=170)
     assert p.returncode == 0, p.stderr[-2000:]
     lines = [ln for ln in p.stdout.splitlines() if ln.strip()]
     assert len(lines) == 1, lines
     d = json.loads(lines[0])
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
-                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "two_launches", "cold",
+                "workloads", "workloads_geomean", "moe_layer"):
         assert key in d, key
+    # the form that runs around a real expert, the cold-cache protocol of the reference's harness, every
+    # named workload and the expert layer are part of the one line
+    assert d["two_launches"]["dispatch_combine_us"] >= d["dispatch_combine_us"] - 0.5
+    assert 0 < d["cold"]["pct_of_hbm_peak"] < 100 and d["cold"]["steps"] <= 30
+    assert set(d["workloads"]) == {"tiny", "dsv3_rank", "skew_world", "fp8_dispatch", "prefill_graph"}
+    for name, w in d["workloads"].items():
+        assert 0 < w["pct_of_hbm_peak"] < 100 and 0 < w["roofline_frac"] < 1 and w["launches_per_step"] >= 1, name
+        assert w["ms_per_step"] * 1e3 >= w["dispatch_combine_us"] - 0.01, name
+        if name != "dsv3_rank":
+            assert w["gpu_output_bit_identical"] is True, name
+    assert d["workloads"]["dsv3_rank"]["dispatch_combine_us"] == d["dispatch_combine_us"]
+    m = d["moe_layer"]
+    assert m["combine_bit_identical_to_oracle_on_gpu_expert_rows"] is True
+    assert m["expert_rows_worst_error_of_tolerance"] <= 1.0 and m["experts_checked"] >= 1
+    assert m["wall_us_per_step"] >= m["expert_gemm"]["us"]
     assert d["n_gpus"] == 1 and d["steps"] == 20 and d["warmup"] == 4
     assert d["unit"] == "GB/s" and d["higher_is_better"] is True and d["vs_baseline"] is None
     assert d["data"] == "synthetic" and d["dtype"] == "bf16"
