@@ -75,8 +75,11 @@ class HipGemmReduceScatter:
     """``forward(input[W, M, Kl], weight[W, N, Kl], bias)`` -> ``out[M, N]``; ``out[r*M/W:(r+1)*M/W]``
     is what rank r of the reference returns."""
 
-    def __init__(self, world_size: int):
+    def __init__(self, world_size: int, pad_ragged: bool = True):
         self.world_size = int(world_size)
+        # False: a shape whose workspace is optional (ragged shards on 256 x 256 tiles, which run faster on
+        # a zero-padded, line-aligned copy of the operands) is multiplied in place, without it
+        self.pad_ragged = bool(pad_ragged)
         self.lib = _lib.load()
         self._workspace = None
 
@@ -104,11 +107,15 @@ class HipGemmReduceScatter:
             raise ValueError(f"bias must be [{N}]")
         if out is None:
             out = torch.empty((M, N), dtype=x.dtype, device=x.device)
-        ws = self.workspace_for(M, N, Kl * W, x.device)
-        rc = self.lib.gemm_rs_forward(
-            x.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, Kl * W, W,
-            0, 0, _lib.BF16 if x.dtype == torch.bfloat16 else _lib.F16, ws.data_ptr() if ws is not None else None,
-            ws.numel() if ws is not None else 0, torch.cuda.current_stream(x.device).cuda_stream)
+        def call(ws):
+            return self.lib.gemm_rs_forward(
+                x.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, Kl * W,
+                W, 0, 0, _lib.BF16 if x.dtype == torch.bfloat16 else _lib.F16, ws.data_ptr() if ws is not None else None,
+                ws.numel() if ws is not None else 0, torch.cuda.current_stream(x.device).cuda_stream)
+
+        rc = call(None) if not self.pad_ragged else -4
+        if rc == -4:  # MOE_A2A_E_WORKSPACE: this shape's form needs its workspace (nothing was launched)
+            rc = call(self.workspace_for(M, N, Kl * W, x.device))
         _lib.check(rc, "gemm_rs_forward")
         return out
 
