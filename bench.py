@@ -960,11 +960,12 @@ def gemm_rs_leg(args, lib, torch, dev):
                     unit="TFLOP/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 5),
                     higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
                     config=dict(workload="gemm_rs", m=m, n=n, k=k, emulated_ranks=W, has_bias=spec["has_bias"],
-                                kernel=kernel, partial_products_workspace_bytes=ws),
+                                kernel=kernel, workspace_bytes=ws),
                     kernels_us=summarise(per), kernel_us=round(t_us, 2),
                     reference_speed_of_light_us_per_gpu_of_8=sol_us.get((m, n, k)))
-        # operands cross HBM once; partial products of the split form are written and read once more
-        gemm_bytes = (m + n) * k * 2 + m * n * 2 + 2 * ws
+        # algorithmic bytes: operands in and the result out, once (what a split form writes and reads again
+        # as partial products, or a padded copy, is the implementation's own traffic and earns nothing)
+        gemm_bytes = (m + n) * k * 2 + m * n * 2
         if gemm_bytes / (HBM_PEAK_GBPS * 1e3) > flops / (MFMA_PEAK_TFLOPS * 1e6):
             gbps = gemm_bytes / t_us / 1e3
             line["roofline"] = dict(bound="hbm", achieved=round(gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",

@@ -82,13 +82,14 @@ enum KernelId {
   KID_GEMM_RS_TILE,
   KID_GEMM_RS_REDUCE,
   KID_GEMM_RS_PAD,
+  KID_GEMM_RS_NARROW,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
     "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token", "forward_tile", "dispatch_fold",
-    "gemm_rs_wide", "gemm_rs_tile", "gemm_rs_reduce", "gemm_rs_pad"};
+    "gemm_rs_wide", "gemm_rs_tile", "gemm_rs_reduce", "gemm_rs_pad", "gemm_rs_narrow"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
