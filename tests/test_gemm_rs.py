@@ -137,7 +137,12 @@ def test_host_side_argument_checks():
     assert need == 8 * 64 * 7168 * 4
     assert call(M=64, N=7168, K=18432) == E_WORKSPACE
     assert call(M=64, N=7168, K=18432, ws=A, wsb=need - 1) == E_WORKSPACE
-    assert lib.gemm_rs_workspace_bytes(8192, 8192, 29568, 8) == 0
+    assert lib.gemm_rs_workspace_bytes(8192, 4096, 14336, 8) == 0  # whole slabs per shard, enough tiles
+    # ragged shards on 256 x 256 tiles: room for both operands in rows padded to whole 64-column slabs
+    # (optional: without it the product runs on the rows as they lie)
+    assert lib.gemm_rs_workspace_bytes(8192, 8192, 29568, 8) == 8 * (8192 + 8192) * 3712 * 2
+    # a few hundred rows: 256 x 128 tiles with the shards in four groups
+    assert lib.gemm_rs_workspace_bytes(512, 4096, 12288, 8) == 4 * 512 * 4096 * 4
     assert lib.gemm_rs_workspace_bytes(64, 64, 100, 8) == 0  # invalid shape: no size
 
 
