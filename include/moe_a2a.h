@@ -383,7 +383,8 @@ const char* moe_a2a_kernel_name(int kernel_id);
 #define MOE_A2A_OPT_TIMER_EVENT_FLAGS 5 /* hipEventCreateWithFlags value for the launch timer's events    */
 #define MOE_A2A_OPT_COMBINE_PLAIN_MAP 6 /* 1: combine workgroups in token order, not grouped by XCD          */
 #define MOE_A2A_OPT_TWO_LAUNCHES 7      /* 1: moe_a2a_forward never takes its one-launch form                */
-#define MOE_A2A_OPT_COUNT 8
+#define MOE_A2A_OPT_FP8_TILE 8          /* tokens per workgroup of the fused routing + fp8 dispatch (0: chosen) */
+#define MOE_A2A_OPT_COUNT 9
 int moe_a2a_set_option(int option, int value);
 int moe_a2a_get_option(int option);
 

@@ -15,7 +15,7 @@ FP8_SCALE_F32, FP8_SCALE_POW2 = 0, 1
 STATUS_BAD_EXPERT, STATUS_OVERFLOW = 1, 2  # bits of the routing status word
 # option switches of moe_a2a_set_option (0 = the library decides)
 (OPT_ROUTE_TILE, OPT_GEMM_TILE, OPT_GEMM_STAGED, OPT_COMBINE_LANES, OPT_COMBINE_VPL, OPT_TIMER_EVENT_FLAGS,
- OPT_COMBINE_PLAIN_MAP, OPT_TWO_LAUNCHES) = range(8)
+ OPT_COMBINE_PLAIN_MAP, OPT_TWO_LAUNCHES, OPT_FP8_TILE) = range(9)
 
 _i32p = C.c_void_p  # device pointers travel as plain addresses
 _vp = C.c_void_p

@@ -12,6 +12,7 @@
 //   dispatch_rows      token row -> K destination rows (read once, store K times)
 //   route_dispatch     both of the above in one launch for small worlds
 //   dispatch_fp8       same copy with e4m3fn quantisation per 128 columns
+//   route_dispatch_fp8 routing and that copy in one launch, a tile of tokens per workgroup
 //   stub_*             expert stand-in, one factor per row
 //   combine / stub_combine   gather K rows per token, weighted sum
 //   forward_token / forward_tile   the whole path of a token (routing, dispatch, stub, weighted sum)
@@ -83,13 +84,14 @@ enum KernelId {
   KID_GEMM_RS_REDUCE,
   KID_GEMM_RS_PAD,
   KID_GEMM_RS_NARROW,
+  KID_ROUTE_DISPATCH_FP8,
   KID_COUNT
 };
 const char* const kKernelNames[KID_COUNT] = {
     "route_tiles", "route_hist", "route_scan", "route_rank",   "dispatch_rows", "route_dispatch", "route_dispatch_tile",
     "dispatch_fp8", "stub_rows",  "stub_fp8",   "combine_rows", "stub_combine", "expert_gemm",
     "expert_gemm_wide", "expert_gemm_skinny", "expert_gemm_f8", "expert_gemm_mx", "route_empty", "forward_token", "forward_tile", "dispatch_fold",
-    "gemm_rs_wide", "gemm_rs_tile", "gemm_rs_reduce", "gemm_rs_pad", "gemm_rs_narrow"};
+    "gemm_rs_wide", "gemm_rs_tile", "gemm_rs_reduce", "gemm_rs_pad", "gemm_rs_narrow", "route_dispatch_fp8"};
 
 // ---------------------------------------------------------------------------------------
 // element helpers: two 16-bit values per dword, element 0 in the low half
@@ -607,6 +609,57 @@ int moe_a2a_dispatch_fp8(const void* x, int x_type, const int32_t* slot_of_entry
 #undef FP8_LAUNCH
 }
 
+// Routing and the fp8 dispatch in one launch (route_dispatch_fp8_tile_kernel), for moe_a2a_forward: any
+// table a tile kernel takes.  Every workgroup counts the whole table for itself, so the launch saves the
+// launch boundary and the index arrays' round trip through memory, not the table pass: 56.1 against
+// 9.4 + 48.5 us at 4096 tokens, top-8, 256 experts, H = 7168.  Tokens per workgroup: tiles of at most 64
+// entries keep the slot arithmetic inside one wave (8 tokens of top-8: 56.1 us; 4: 57.9, 16: 62.5, 32:
+// 79.5); more tokens per tile only beyond two workgroups per CU.
+static bool route_dispatch_fp8_ok(int T, int K, int H) {
+  return T > 0 && K <= kTileMaxOwn && H % MOE_A2A_FP8_BLOCK == 0;
+}
+static int fp8_tile_tokens(int T, int K) {
+  const int cap = std::max(kTileMaxOwn / K, 1), wave = std::max(kWave / K, 1);
+  const int forced = option(MOE_A2A_OPT_FP8_TILE);
+  if (forced > 0) return std::min(forced, cap);
+  return std::min(cap, std::max(wave, ceil_div(T, 2 * 256)));
+}
+static int route_dispatch_fp8_impl(const void* x, int x_type, const int32_t* indices, const int32_t* rank_start,
+                                   int src_rank, int T, int K, int E, int W, int H, int max_recv, int32_t* counts,
+                                   int32_t* offsets, int32_t* slot_of_entry, int32_t* src_of_slot, int32_t* meta,
+                                   int32_t* status, void* disp_q, float* disp_scale, int pow2, hipStream_t stream,
+                                   int32_t* clear_status) {
+  if (int rc = check_route_shape(T, K, E, W)) return rc;
+  if (max_recv < 0 || (long long)max_recv * E > (long long)INT32_MAX / 8) return MOE_A2A_E_SHAPE;
+  if (int rc = check_rows(x, disp_q, T, K, H, MOE_A2A_FP8_BLOCK)) return rc;
+  if (!counts || !offsets || !indices || !slot_of_entry || !src_of_slot || !meta || !disp_scale) return MOE_A2A_E_NULL;
+  RouteArgs a{indices, rank_start, src_rank, T, K, E, W, T * K, id_bits(E), max_recv, counts, offsets,
+              slot_of_entry, src_of_slot, meta, status, clear_status};
+  const int nblk = H / MOE_A2A_FP8_BLOCK;
+  const int tile = fp8_tile_tokens(T, K);
+  // workgroups of 512 lanes, three to a CU, so that one's table pass runs under another's rows (a thread
+  // per expert in the scan: 1024 lanes beyond 512 experts)
+  const int threads = E <= 512 ? 512 : kTileThreads;
+  dim3 grid((unsigned)ceil_div(T, tile)), block(threads);
+  const bool st = streams(T, (long long)T * K, H, 2, 1);
+#define RDF8_T(EL, ST, TH)                                                                                       \
+  return launch(KID_ROUTE_DISPATCH_FP8, route_dispatch_fp8_tile_kernel<EL, ST, TH>, grid, block, 0, stream, a,   \
+                (const uint4*)x, (uint4*)disp_q, disp_scale, nblk, tile, pow2)
+#define RDF8(EL, ST)                         \
+  {                                          \
+    if (threads == 512) RDF8_T(EL, ST, 512); \
+    RDF8_T(EL, ST, kTileThreads);            \
+  }
+  if (x_type == MOE_A2A_BF16) {
+    if (st) RDF8(Bf16, 1);
+    RDF8(Bf16, 0);
+  }
+  if (st) RDF8(F16, 1);
+  RDF8(F16, 0);
+#undef RDF8_T
+#undef RDF8
+}
+
 static bool known_type(int t) { return t == MOE_A2A_F16 || t == MOE_A2A_BF16; }
 
 int moe_a2a_stub(const void* disp, const float* disp_scale, const int32_t* meta, const int32_t* rows, int in_type,
@@ -836,9 +889,10 @@ static bool dispatch_fold_ok(int T, int K, int H, int max_recv, int in_type, int
                              int fuse_route) {
   if (max_recv > 0 || in_type != out_type || T < 1) return false;
   if (option(MOE_A2A_OPT_TWO_LAUNCHES) == 1) return false;
-  // The fp8 dispatch is always routed by a launch of its own.  The fold behind it pays while the rows
-  // stay in the caches (one launch boundary less); at streaming volumes the two separate kernels move
-  // the same bytes about 1 % faster (120.0 against 118.8 us at 16384 tokens, top-8, H = 7168).
+  // The fold behind an fp8 dispatch is routed by a launch of its own.  It pays while the rows stay in
+  // the caches (one launch boundary less); at streaming volumes two kernels (routing + dispatch in one,
+  // then stub + combine) move the same bytes about 1 % faster (120.0 against 118.8 us at 16384 tokens,
+  // top-8, H = 7168).
   if (fp8_dispatch) return !streams(T, 2ll * T * K, H, 2, 1);
   return !(fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
 }
@@ -926,7 +980,8 @@ int moe_a2a_forward_launches(int T, int K, int H, int max_recv, int in_type, int
     if (R <= kRouteTilesMaxRows) return 2;
     return ceil_div((int)std::min<long long>(R, INT32_MAX), kRouteThreads) <= kRouteFoldMaxTiles ? 3 : 4;
   }
-  const bool fused = !fp8_dispatch && (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
+  const bool fused = fp8_dispatch ? (fuse_route && route_dispatch_fp8_ok(T, K, H))
+                                  : (fuse_route == 2 ? K <= kTileMaxOwn : (fuse_route == 1 && moe_a2a_fused_ok(T, K, H)));
   int n = fused ? 1 : 2;  // routing + dispatch
   if (!fused) {
     const long long R = (long long)T * K;
@@ -1040,6 +1095,11 @@ static int forward_impl(const void* x, const int32_t* indices, const float* weig
   if (fused) {
     if (int rc = route_dispatch_impl(x, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts, offsets,
                                      slot_of_entry, src_of_slot, meta, status, disp, stream, clear_status))
+      return rc;
+  } else if (fp8_dispatch && fuse_route && route_dispatch_fp8_ok(T, K, H)) {
+    if (int rc = route_dispatch_fp8_impl(x, in_type, indices, rank_start, src_rank, T, K, E, W, H, max_recv, counts,
+                                         offsets, slot_of_entry, src_of_slot, meta, status, disp, disp_scale,
+                                         fp8_dispatch == 2, (hipStream_t)stream, clear_status))
       return rc;
   } else {
     if (int rc = route_impl(indices, rank_start, src_rank, T, K, E, W, max_recv, counts, offsets, slot_of_entry,

@@ -421,6 +421,83 @@ def test_forward_with_fp8_dispatch_and_folded_stub(gpu_device, options, W, E, K,
             assert_same(f"{key} ({'separate launches' if two else 'one kernel'})", val, want[key])
 
 
+@pytest.mark.parametrize("W,E,K,H,tokens", [
+    (1, 8, 2, 128, [1]),                              # one token, one block
+    (8, 256, 8, 7168, [40, 0, 3, 0, 17, 0, 0, 1]),
+    (2, 16, 3, 384, [2001, 1000]),                    # 9003 entries: past the first table batch, R % 4 = 3
+    (4, 64, 8, 1024, [1200, 0, 900, 1011]),           # 24888 entries: the vector pass over the table
+    (2, 32, 5, 2048, [33, 20]),                       # K = 5: tiles of 12 tokens, the last one short
+])
+@pytest.mark.parametrize("fp8", [True, "pow2"], ids=["f32scales", "pow2scales"])
+@pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
+def test_forward_routes_and_quantises_in_one_launch(gpu_device, options, W, E, K, H, tokens, fp8, padded):
+    """forward with an fp8 dispatch routes and quantises in one launch (a tile of tokens per
+    workgroup): index arrays, rows, scales and output bit for bit those of the oracle and of the
+    routing launch followed by dispatch_fp8, at the chosen tile and at forced tiles of 1, 5 and 32 tokens."""
+    g = torch.Generator().manual_seed(sum(tokens) + E + K)
+    dtype = torch.bfloat16 if K % 2 else torch.float16
+    cfg = C.MoEConfig(E, K, H, max(tokens) + 1, dtype, dtype)
+    world = []
+    for n in tokens:
+        idx = (torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(n)]).to(torch.int32) if n
+               else torch.empty(0, K, dtype=torch.int32))
+        world.append(C.RankData(n, idx, torch.rand(n, K, generator=g), torch.randn(n, H, generator=g).to(dtype)))
+    x, idx, w, rs = concat_world(world, gpu_device)
+    T = x.shape[0]
+    want = V.run_world(cfg, world, stub_kind=C.STUB_EXPERT_FRACTION, fp8=True, pow2=fp8 == "pow2")
+    lib = _lib.load()
+    elem = _lib.BF16 if dtype == torch.bfloat16 else _lib.F16
+    assert lib.moe_a2a_forward_launches(T, K, H, 0, elem, elem, 1, 1, 0) == 3
+    assert lib.moe_a2a_forward_launches(T, K, H, 0, elem, elem, 1, 0, 0) == (4 if T * K <= 32768 else 5)
+    ref = None
+    for fuse_route, tile in ((False, 0), (True, 0), (True, 1), (True, 5), (True, 32)):
+        options.set("FP8_TILE", tile)
+        ata = HipAllToAll(cfg, 0, W, stub_kind=C.STUB_EXPERT_FRACTION, fp8_dispatch=fp8, fuse_route=fuse_route,
+                          fuse_stub=False, padded=padded)
+        for _ in range(2):
+            y = ata.forward(x, idx, w, rs)
+        torch.cuda.synchronize()
+        d = ata.last
+        assert int(d.status.item()) == 0
+        what = f"route_dispatch_fp8, tile {tile}" if fuse_route else "separate launches"
+        got = dict(counts=d.counts, offsets=d.offsets, slot_of_entry=d.slot_of_entry, src_of_slot=d.src_of_slot,
+                   meta=d.meta, disp_x=d.disp_x, disp_scale=d.disp_scale, y=y)
+        if not padded:
+            for key, val in got.items():
+                assert_same(f"{key} ({what})", val, want[key])
+        else:  # the padded layout against the compact one: entry by entry, and the output
+            assert_same(f"counts ({what})", d.counts, want["counts"])
+            assert_same(f"y ({what})", y, want["y"])
+            slots, wslots = d.slot_of_entry.cpu().long().flatten(), want["slot_of_entry"].long().flatten()
+            assert torch.equal(d.disp_x.cpu()[slots], want["disp_x"][wslots])
+            assert torch.equal(bits(d.disp_scale.cpu()[slots]), bits(want["disp_scale"][wslots]))
+            assert torch.equal(d.meta.cpu()[slots], want["meta"][wslots])
+        if ref is None:
+            ref = {k: v.clone() for k, v in got.items()}
+        else:  # rows no entry owns are not written by either form: compare what the entries own
+            for key in ("counts", "offsets", "slot_of_entry", "y"):
+                assert torch.equal(bits(got[key]), bits(ref[key])), f"{key} ({what})"
+    # the launch timer names the kernel
+    import ctypes
+    options.set("FP8_TILE", 0)
+    assert lib.moe_a2a_timer_begin(8) == 0
+    ata.forward(x, idx, w, rs)
+    ids, us = (ctypes.c_int * 8)(), (ctypes.c_float * 8)()
+    assert lib.moe_a2a_timer_end(ids, us, 8) == 3
+    assert lib.moe_a2a_kernel_name(ids[0]) == b"route_dispatch_fp8"
+
+
+def test_one_launch_fp8_routing_reports_a_bad_expert_id(gpu_device):
+    cfg = C.MoEConfig(16, 2, 256, 64, torch.bfloat16, torch.bfloat16)
+    g = torch.Generator().manual_seed(5)
+    idx = torch.stack([torch.randperm(16, generator=g)[:2] for _ in range(64)]).to(torch.int32)
+    idx[17, 1] = 16
+    x = torch.randn(64, 256, generator=g).to(torch.bfloat16).to(gpu_device)
+    ata = HipAllToAll(cfg, 0, 1, fp8_dispatch=True, fuse_stub=False)
+    with pytest.raises(IndexError):
+        ata.forward(x, idx.to(gpu_device), torch.rand(64, 2, generator=g).to(gpu_device), check_status=True)
+
+
 @pytest.mark.parametrize("name", GOLDEN_CASES)
 @pytest.mark.parametrize("fuse_route", ["always", False])
 def test_padded_layout_is_the_reference_dispatch_return_value(gpu_device, name, fuse_route):
