@@ -122,6 +122,9 @@ def parse_args():
                    help="measure the GEMM + reduce-scatter of the reference's other problem instead (8 emulated ranks "
                         "as K shards of one buffer), e.g. 8192,8192,29568 or 512,4096,12288,bias; `all` runs the six "
                         "benchmark shapes of gemm_rs/task.yml, one JSON line each")
+    p.add_argument("--equal-segments", action="store_true",
+                   help="with --expert-gemm: a routing table that gives every expert the same number of rows "
+                        "(entry i goes to expert i %% E) instead of the workload's")
     p.add_argument("--expert-gemm", type=int, default=0, metavar="N",
                    help="measure the grouped expert GEMM (N output columns per expert) on the workload's "
                         "dispatched rows instead of the dispatch/combine path")
@@ -845,6 +848,8 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
         weights = (wf / w_scale[:, :, None, :, None]).to(torch.float8_e4m3fn).view(E, N, H).contiguous()
     main = torch.cuda.Stream()
     main.wait_stream(torch.cuda.current_stream())
+    if args.equal_segments:
+        idx = (torch.arange(idx.numel(), device=dev, dtype=torch.int32) % E).view_as(idx).contiguous()
     with torch.cuda.stream(main):
         d = ata.dispatch(x, idx, rs)
         R = d.num_rows
@@ -870,6 +875,7 @@ def expert_gemm_leg(args, lib, torch, wl, x, idx, rs, dev):
                scaling="weak", vs_baseline=None, dtype="bf16" if cfg.in_dtype == torch.bfloat16 else "f16",
                data="synthetic",
                config=dict(workload=wl.name + "+expert_gemm", rows=R, experts=E, hidden=H, out_columns=N, kernel=kernel,
+                           segments="equal" if args.equal_segments else "the workload's routing",
                            rows_dtype="fp8 e4m3fn + f32 scale per 128 columns" if fp8 else "16-bit",
                            weights_dtype="fp8 e4m3fn + f32 scale per 128 x 128 block" if args.fp8_weights else "16-bit"),
                kernels_us=summarise(per),
