@@ -748,7 +748,8 @@ def calibrate_copy(torch, main, dev):
     torch.cuda.synchronize()
 
 
-KERNEL_OF_SYMBOL = (("route_dispatch_tile_kernel", "route_dispatch_tile"), ("route_dispatch_kernel", "route_dispatch"),
+KERNEL_OF_SYMBOL = (("route_dispatch_fp8_tile_kernel", "route_dispatch_fp8"),
+                    ("route_dispatch_tile_kernel", "route_dispatch_tile"), ("route_dispatch_kernel", "route_dispatch"),
                     ("forward_token_kernel", "forward_token"), ("forward_tile_kernel", "forward_tile"),
                     ("dispatch_fold_kernel", "dispatch_fold"),
                     ("stub_combine_rows_kernel", "stub_combine"), ("stub_combine_fp8_kernel", "stub_combine"),
