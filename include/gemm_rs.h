@@ -32,11 +32,21 @@ extern "C" {
  *   bias    [N] of elem_type, or NULL
  *   out     [M, N] of elem_type
  *   K % W == 0, (K/W) % 8 == 0, 16-byte aligned operands; M need not divide by W for the sum itself
- *   workspace  gemm_rs_workspace_bytes(M, N, K, W) bytes, 16-byte aligned (0 bytes for most shapes:
- *           only outputs of few tiles keep one f32 partial product per shard, which a second launch
- *           sums -- what each rank holds before the reduce-scatter); MOE_A2A_E_WORKSPACE if too small
- * The option MOE_A2A_OPT_GEMM_TILE = 256 / 128 / 32 forces the 256 x 256 tiles, the 128 x 128 tiles
- * or the per-shard partial products where the shape allows them.
+ *   workspace  gemm_rs_workspace_bytes(M, N, K, W) bytes, 16-byte aligned; what it is for depends on the
+ *           kernel form the shape gets:
+ *             - outputs of few tiles spread the shards over groups of workgroups, one f32 partial
+ *               product per group (what each rank holds before the reduce-scatter), which a second
+ *               launch sums: REQUIRED, MOE_A2A_E_WORKSPACE if missing or too small;
+ *             - large outputs whose local K is not a multiple of 64 (rows that start off the
+ *               128-byte line grid) are first copied onto zero-padded, aligned rows: OPTIONAL --
+ *               with NULL or too few bytes the product runs on the rows as they lie, about a
+ *               tenth slower;
+ *             - 0 bytes for every other shape.
+ *           The form, and with it the size, follows MOE_A2A_OPT_GEMM_TILE at the time of the call: a
+ *           size queried under one setting belongs to that setting.
+ * MOE_A2A_OPT_GEMM_TILE forces a form where the shape allows it: 256 the 256 x 256 tiles, 129 the
+ * 256 x 128 tiles, 130 those with one partial product per shard, 128 the 128 x 128 tiles, 32 those
+ * with one partial product per shard.  All unsplit forms give identical bits.
  */
 size_t gemm_rs_workspace_bytes(int M, int N, int K, int W);
 int gemm_rs_forward(const void* input, const void* weight, const void* bias, void* out, int M, int N, int K, int W,
