@@ -209,19 +209,16 @@ def test_expert_gemm_block_quantised_weights(gpu_device, options, E, K, T, H, N,
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-@pytest.mark.parametrize("staged", [False, True], ids=["direct", "staged"])
-def test_expert_gemm_power_of_two_scales(gpu_device, options, E, K, T, H, N, W, zipf, dtype, padded, staged):
+@pytest.mark.parametrize("form", [0, 2, 1], ids=["eight", "direct", "staged"])
+def test_expert_gemm_power_of_two_scales(gpu_device, options, E, K, T, H, N, W, zipf, dtype, padded, form):
     """fp8 rows and fp8 weights whose scales are powers of two, multiplied by the fp8 matrix
     instruction with the scales as its block exponents, against the f32 matmul of the
     dequantised operands; the fp8 x fp8 kernel with the fold on the vector units, which takes
-    any f32 scale, has to agree with it to f32 summation order.  Both forms of the tiled kernel:
-    slabs sent memory -> LDS directly (hidden sizes that are multiples of 256) and staged through
-    registers (every hidden size)."""
+    any f32 scale, has to agree with it to f32 summation order.  All forms of the tiled kernel:
+    eight waves on slabs of 128 columns (hidden sizes from 256), four waves with slabs of 64 columns
+    sent memory -> LDS directly (multiples of 256) and staged through registers (every hidden size)."""
     options.set("GEMM_TILE", "256")  # the tiles at every segment length
-    if staged:
-        options.set("GEMM_STAGED", 1)
-    else:
-        options.set("GEMM_STAGED", 0)
+    options.set("GEMM_STAGED", form)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=7 * E + T, zipf=zipf)
     wq, ws = V.quantize_weights_fp8(weights, pow2=True)
     x, idx, w, rs = concat_world(world, gpu_device)
@@ -241,7 +238,7 @@ def test_expert_gemm_power_of_two_scales(gpu_device, options, E, K, T, H, N, W, 
 
 
 @pytest.mark.parametrize("form", ["16bit-32", "16bit-128", "16bit-256", "q8-32", "q8-32staged", "q8-128", "q8-256",
-                                  "mx-direct", "mx-staged"])
+                                  "mx-eight", "mx-direct", "mx-staged"])
 def test_padded_overflow_stays_inside_the_buffers(gpu_device, options, form):
     """Padded layout with a LAST expert that receives more rows than max_recv (routing folds the
     surplus onto the segment's last row and raises the overflow bit; counts stay the true numbers):
@@ -259,6 +256,8 @@ def test_padded_overflow_stays_inside_the_buffers(gpu_device, options, form):
     options.set("GEMM_TILE", int(tile[:3].rstrip("sd")) if tile[0].isdigit() else 256)
     if tile in ("32staged", "staged"):
         options.set("GEMM_STAGED", 1)
+    if tile == "direct":
+        options.set("GEMM_STAGED", 2)
     fp8 = {"16bit": False, "q8": True, "mx": "pow2"}[kind]
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, W, fp8_dispatch=fp8, padded=True, max_recv=max_recv)
