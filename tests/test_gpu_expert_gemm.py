@@ -206,6 +206,8 @@ def test_expert_gemm_block_quantised_weights(gpu_device, options, E, K, T, H, N,
     (8, 2, 1200, 256, 512, 2, False),    # 300 rows per expert
     (3, 1, 1000, 1024, 256, 1, False),   # 333 rows per expert, eight K blocks
     (5, 2, 700, 768, 640, 1, True),      # twelve slabs of 64 bytes, a 128-column tail tile, ragged
+    (2, 1, 300, 8192, 256, 1, False),    # 64 scale blocks per row: the eight-wave form's exponent table is full
+    (2, 1, 300, 8448, 256, 1, False),    # 66: beyond it (the four-wave forms run)
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
