@@ -328,17 +328,19 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
 /*
  * The same product for operands whose scales are all powers of two (rows from moe_a2a_dispatch_fp8
  * with MOE_A2A_FP8_SCALE_POW2, weights quantised with power-of-two block scales, the UE8M0 style
- * of newer DeepSeek checkpoints): the bytes of both operands go to
- * v_mfma_scale_f32_32x32x64_f8f6f4 and the exponent fields of the scales ride along as the
- * instruction's block exponents, so the products of all K blocks accumulate inside the matrix
- * cores (256 x 256 tiles, nothing is folded on the vector units; with Kd % 256 == 0 the operand
- * slabs travel memory -> LDS directly, three slabs ahead).  y = sum over K blocks of
+ * of newer DeepSeek checkpoints): the bytes of both operands go to the scaled fp8 matrix
+ * instruction (v_mfma_scale_f32_16x16x128_f8f6f4 on eight-wave 256 x 256 tiles for Kd from 256 to
+ * 8192; v_mfma_scale_f32_32x32x64_f8f6f4 on four-wave tiles otherwise) and the exponent fields of
+ * the scales ride along as the instruction's block exponents, so the products of all K blocks
+ * accumulate inside the matrix cores (nothing is folded on the vector units; the operand slabs
+ * travel memory -> LDS directly).  y = sum over K blocks of
  * x_scale * w_scale * (q_x . q_w) in f32, one rounding to elem_type.  ONLY the exponent field of a
  * scale is used: a scale that is not a power of two is silently taken as the power of two below
  * it.  Segments of at most 32 rows on average (a decode step), and other Kd on segments shorter
  * than 256 rows, go through moe_a2a_expert_gemm_q8 (any f32 scale).  The option
  * MOE_A2A_OPT_GEMM_TILE = 256 forces the tiles, 32 / 128 the kernels of moe_a2a_expert_gemm_q8,
- * MOE_A2A_OPT_GEMM_STAGED = 1 the register-staged loop of the tiles.  Arguments as for
+ * MOE_A2A_OPT_GEMM_STAGED = 1 the register-staged four-wave loop of the tiles, 2 the four-wave loop
+ * with slabs sent memory -> LDS (Kd % 256 == 0).  Arguments as for
  * moe_a2a_expert_gemm_q8 with x_scale required.  No counterpart in the reference.
  */
 int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w_q, const float* w_scale,
@@ -377,7 +379,8 @@ const char* moe_a2a_kernel_name(int kernel_id);
  */
 #define MOE_A2A_OPT_ROUTE_TILE 0    /* 1: moe_a2a_route_dispatch takes the token-tile kernel at any size   */
 #define MOE_A2A_OPT_GEMM_TILE 1     /* 32 | 128 | 256: tile family of the expert GEMM entry points          */
-#define MOE_A2A_OPT_GEMM_STAGED 2   /* 1: register-staged form of the weight-streaming / scaled-MFMA loops  */
+#define MOE_A2A_OPT_GEMM_STAGED 2   /* 1: register-staged form of the weight-streaming / scaled-MFMA loops;
+                                       2: four-wave direct form of moe_a2a_expert_gemm_mx8                  */
 #define MOE_A2A_OPT_COMBINE_LANES 3 /* lanes of a combine workgroup at cache-resident sizes (64 .. 512)     */
 #define MOE_A2A_OPT_COMBINE_VPL 4   /* 2: two row vectors per lane in the combine at cache-resident sizes   */
 #define MOE_A2A_OPT_TIMER_EVENT_FLAGS 5 /* hipEventCreateWithFlags value for the launch timer's events    */
