@@ -176,12 +176,13 @@ def test_empty_world_never_reaches_a_kernel_that_reads_the_table(lib):
 
 
 def test_option_switches(lib):
-    for opt in range(8):
+    n_options = _lib.OPT_FP8_TILE + 1  # the last one
+    for opt in range(n_options):
         assert lib.moe_a2a_get_option(opt) == 0  # nothing is on unless a caller turns it on
     assert lib.moe_a2a_set_option(_lib.OPT_GEMM_TILE, 128) == 0
     assert lib.moe_a2a_get_option(_lib.OPT_GEMM_TILE) == 128
     assert lib.moe_a2a_set_option(_lib.OPT_GEMM_TILE, 0) == 128  # returns the previous value
-    assert lib.moe_a2a_set_option(-1, 1) == E_DTYPE and lib.moe_a2a_set_option(8, 1) == E_DTYPE
+    assert lib.moe_a2a_set_option(-1, 1) == E_DTYPE and lib.moe_a2a_set_option(n_options, 1) == E_DTYPE
     assert lib.moe_a2a_get_option(99) == E_DTYPE
     # no option takes a negative value, so a negative return always means an error
     assert lib.moe_a2a_set_option(_lib.OPT_GEMM_TILE, -3) == E_SHAPE
