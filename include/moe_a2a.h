@@ -311,8 +311,10 @@ int moe_a2a_expert_gemm_fp8(const void* x_q, const float* x_scale, const void* w
  *     both operands go to the fp8 matrix instruction untouched, folded per K block as below.
  *     The option MOE_A2A_OPT_GEMM_STAGED = 1 selects the register-staged form of the same
  *     arithmetic (fp8 rows are then dequantised and rounded once to elem_type first).
- *   longer segments, fp8 rows: both operands enter the fp8 matrix instruction as bytes
- *     (v_mfma_f32_32x32x64_f8f6f4), each 128-wide K block is summed in f32 and folded with
+ *   longer segments, fp8 rows: both operands enter the fp8 matrix instruction as bytes (eight
+ *     waves on 256 x 128 tiles with the 16x16x128 instruction for Kd >= 256; the option
+ *     MOE_A2A_OPT_GEMM_STAGED = 2, and Kd = 128, take four waves on 128 x 128 tiles with the
+ *     32x32x64 one), each 128-wide K block is summed in f32 and folded with
  *     x_scale[row][kb] * w_scale[n / 128][kb]; nothing is rounded before the output.
  *   longer segments, 16-bit rows (and N >= 256): the 256 x 256 kernel; a weight enters the matrix
  *     cores as elem(f32(q) * scale), i.e. dequantised and rounded once to elem_type on its way into
@@ -380,7 +382,7 @@ const char* moe_a2a_kernel_name(int kernel_id);
 #define MOE_A2A_OPT_ROUTE_TILE 0    /* 1: moe_a2a_route_dispatch takes the token-tile kernel at any size   */
 #define MOE_A2A_OPT_GEMM_TILE 1     /* 32 | 128 | 256: tile family of the expert GEMM entry points          */
 #define MOE_A2A_OPT_GEMM_STAGED 2   /* 1: register-staged form of the weight-streaming / scaled-MFMA loops;
-                                       2: four-wave direct form of moe_a2a_expert_gemm_mx8                  */
+                                       2: four-wave forms of moe_a2a_expert_gemm_mx8 / _q8 with fp8 rows    */
 #define MOE_A2A_OPT_COMBINE_LANES 3 /* lanes of a combine workgroup at cache-resident sizes (64 .. 512)     */
 #define MOE_A2A_OPT_COMBINE_VPL 4   /* 2: two row vectors per lane in the combine at cache-resident sizes   */
 #define MOE_A2A_OPT_TIMER_EVENT_FLAGS 5 /* hipEventCreateWithFlags value for the launch timer's events    */
