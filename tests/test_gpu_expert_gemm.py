@@ -166,11 +166,14 @@ def test_decode_shape_takes_the_skinny_kernel(gpu_device, options):
     (64, 4, 128, 512, 384, 8, False),    # decode-like: 8 rows per expert
     (16, 4, 300, 384, 256, 4, True),     # skewed: empty experts and long segments
     (8, 2, 1200, 256, 256, 2, False),    # 300 rows per expert
+    (4, 2, 1100, 1024, 384, 1, True),    # eight K blocks, three 128-column tiles, long ragged segments
+    (3, 1, 700, 640, 128, 1, False),     # five K blocks: the three-buffer loop ends on its second tail step
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("fp8_rows", [False, True], ids=["rows16", "rows8"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-@pytest.mark.parametrize("tile", ["32", "32r", "128", "256"], ids=["tile32", "tile32staged", "tile128", "tile256"])
+@pytest.mark.parametrize("tile", ["32", "32r", "128", "128f", "256"],
+                         ids=["tile32", "tile32staged", "tile128", "tile128fourwaves", "tile256"])
 def test_expert_gemm_block_quantised_weights(gpu_device, options, E, K, T, H, N, W, zipf, dtype, fp8_rows,
                                              padded, tile):
     """Weights as e4m3fn bytes with one scale per 128 x 128 block, rows 16-bit or from the fp8
@@ -179,9 +182,11 @@ def test_expert_gemm_block_quantised_weights(gpu_device, options, E, K, T, H, N,
     128, fp8 rows only: 16-bit rows keep the default choice) and the 256 x 256 kernel (which needs
     N >= 256; the one N == 128 case stays on the other).  The weight-streaming form exists twice:
     slabs sent memory -> LDS directly (tile32) and staged through registers (tile32staged)."""
-    options.set("GEMM_TILE", tile[:2] if tile.startswith("32") else tile)
+    options.set("GEMM_TILE", tile[:2] if tile.startswith("32") else tile[:3])
     if tile == "32r":
         options.set("GEMM_STAGED", 1)
+    if tile == "128f":  # the four-wave 128 x 128 form of the fp8 x fp8 kernel (eight waves on 256 x 128 otherwise)
+        options.set("GEMM_STAGED", 2)
     cfg, world, weights = make(E, K, T, H, N, W, dtype, seed=5 * E + T, zipf=zipf)
     wq, ws = V.quantize_weights_fp8(weights)
     x, idx, w, rs = concat_world(world, gpu_device)
@@ -192,7 +197,7 @@ def test_expert_gemm_block_quantised_weights(gpu_device, options, E, K, T, H, N,
     o = V.run_world(cfg, world, fp8=fp8_rows)
     # fp8 rows on segments of more than 32 rows take the fp8 x fp8 kernel unless another is forced: no
     # rounding of the rows there
-    f8_kernel = fp8_rows and (tile == "128" or (tile == "256" and N < 256 and d.num_rows > 32 * E))
+    f8_kernel = fp8_rows and (tile in ("128", "128f") or (tile == "256" and N < 256 and d.num_rows > 32 * E))
     want = V.expert_gemm_q8(o["disp_x"], o["disp_scale"] if fp8_rows else None, wq, ws, o["offsets"], dtype,
                             round_rows=not f8_kernel)
     rows = d.slot_of_entry.long() if padded else o["slot_of_entry"].long().to(gpu_device)
