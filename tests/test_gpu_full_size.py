@@ -70,6 +70,36 @@ def test_full_size_against_oracle(gpu_device, name):
                 assert torch.equal(bits(y3.cpu()), bits(want32))
 
 
+@pytest.mark.parametrize("fp8", [True, "pow2"], ids=["f32scales", "pow2scales"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_fp8_forward_routes_and_quantises_in_one_launch_at_full_size(gpu_device, fp8, dtype):
+    """The fp8 workload through forward (routing + fp8 dispatch in one launch, then stub + combine): index
+    arrays, rows, scales and output bit for bit the oracle's, for both scale modes and both element types."""
+    import dataclasses
+
+    from kernel_amd import _lib
+
+    wl = C.generate_workload("fp8_dispatch")
+    cfg = dataclasses.replace(wl.cfg, in_dtype=dtype, out_dtype=dtype)
+    world = [C.RankData(r.num_tokens, r.indices, r.weights, r.x.to(dtype)) for r in wl.world]
+    want = V.run_world(cfg, world, stub_kind=wl.stub_kind, fp8=True, pow2=fp8 == "pow2", combine_mode=C.COMBINE_F32)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    T, K, H = x.shape[0], cfg.experts_per_token, cfg.hidden_dim
+    elem = _lib.BF16 if dtype == torch.bfloat16 else _lib.F16
+    assert _lib.load().moe_a2a_forward_launches(T, K, H, 0, elem, elem, 2 if fp8 == "pow2" else 1, 1, 1) == 2
+    ata = HipAllToAll(cfg, 0, wl.world_size, stub_kind=wl.stub_kind, combine_mode=C.COMBINE_F32, fp8_dispatch=fp8,
+                      fuse_stub=True)
+    for _ in range(2):  # both buffer sets
+        y = ata.forward(x, idx, w, rs)
+        torch.cuda.synchronize()
+        d = ata.last
+        assert int(d.status.item()) == 0
+        for key in ("counts", "offsets", "slot_of_entry", "src_of_slot", "meta", "disp_x"):
+            assert torch.equal(bits(getattr(d, key).cpu()), bits(want[key])), key
+        assert torch.equal(bits(d.disp_scale.cpu()), bits(want["disp_scale"]))
+        assert torch.equal(bits(y.cpu()), bits(want["y"]))
+
+
 def test_fp8_rows_within_stated_bound_at_full_size(gpu_device):
     """After dequantisation: |q*scale - x| <= max(2^-4 |x|, 2^-10 scale) for every element."""
     wl = C.generate_workload("fp8_dispatch")
