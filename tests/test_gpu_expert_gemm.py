@@ -422,3 +422,57 @@ def test_random_shapes_every_expert_gemm_form(gpu_device, options, seed):
     torch.cuda.synchronize()
     rows = d.slot_of_entry.long() if padded else o["slot_of_entry"].long().to(gpu_device)
     close(y[rows], want[o["slot_of_entry"].long()])
+
+
+def make_counts(counts, H, N, dtype, seed):
+    """One rank, one expert per token, expert e receiving exactly counts[e] rows (shuffled)."""
+    g = torch.Generator().manual_seed(seed)
+    E = len(counts)
+    ids = torch.repeat_interleave(torch.arange(E), torch.tensor(counts))
+    ids = ids[torch.randperm(ids.numel(), generator=g)].to(torch.int32).reshape(-1, 1)
+    T = ids.shape[0]
+    cfg = C.MoEConfig(E, 1, H, T + 1, dtype, dtype)
+    world = [C.RankData(T, ids, torch.rand(T, 1, generator=g), torch.randn(T, H, generator=g).to(dtype))]
+    weights = (torch.randn(E, N, H, generator=g) / H ** 0.5).to(dtype)
+    return cfg, world, weights
+
+
+def walk_cases():
+    lone = [0, 0, 0, 3500, 0]                       # fourteen m-tiles of one expert: several groups of four
+    gaps = [0] * 64
+    for e, n in ((1, 256), (2, 257), (17, 1025), (18, 1), (40, 255), (63, 513)):
+        gaps[e] = n                                 # tile-exact, one past a tile, one row, runs of empty experts
+    many = [0] * 1024
+    for e in range(0, 1024, 3):
+        many[e] = 1 + (e * 7) % 5                   # the largest expert count: a few rows on every third
+    many[1023] = 700
+    ends = [300] + [0] * 30 + [300]                 # rows only on the first and the last expert
+    return [("lone", lone), ("gaps", gaps), ("many", many), ("ends", ends)]
+
+
+@pytest.mark.parametrize("name,counts", walk_cases(), ids=[c[0] for c in walk_cases()])
+@pytest.mark.parametrize("fmt", ["16bit", "mx", "f32scale"])
+@pytest.mark.parametrize("N", [256, 640])
+def test_eight_wave_tile_walk_on_odd_segment_tables(gpu_device, options, name, counts, fmt, N):
+    """The eight-wave kernels give every expert's m-tiles to one die's workgroups, in groups of at
+    most four.  Segment tables that stress that walk: one expert with many tiles, tile-exact and
+    one-row segments between runs of empty experts, the largest expert count, rows only at the two
+    ends; one n-tile and a ragged last n-tile; each operand format's eight-wave kernel forced."""
+    dtype, H = torch.bfloat16, 256
+    options.set("GEMM_TILE", "128" if fmt == "f32scale" else "256")
+    cfg, world, weights = make_counts(counts, H, N, dtype, seed=len(counts) + N)
+    x, idx, w, rs = concat_world(world, gpu_device)
+    fp8 = {"16bit": False, "mx": "pow2", "f32scale": True}[fmt]
+    ata = HipAllToAll(cfg, 0, 1, fp8_dispatch=fp8)
+    d = ata.dispatch(x, idx, rs)
+    o = V.run_world(cfg, world, fp8=bool(fp8), pow2=fmt == "mx")
+    assert o["offsets"].tolist() == torch.tensor([0] + counts).cumsum(0).tolist()
+    if fmt == "16bit":
+        y = ata.expert_gemm(d, weights.to(gpu_device))
+        want = V.expert_gemm(o["disp_x"], o["offsets"], weights, dtype)
+    else:
+        wq, ws = V.quantize_weights_fp8(weights, pow2=fmt == "mx")
+        y = ata.expert_gemm(d, wq.to(gpu_device), w_scale=ws.to(gpu_device), scales_pow2=fmt == "mx")
+        want = V.expert_gemm_q8(o["disp_x"], o["disp_scale"], wq, ws, o["offsets"], dtype, round_rows=False)
+    torch.cuda.synchronize()
+    close(y, want)
