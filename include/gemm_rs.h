@@ -45,8 +45,9 @@ extern "C" {
  *           The form, and with it the size, follows MOE_A2A_OPT_GEMM_TILE at the time of the call: a
  *           size queried under one setting belongs to that setting.
  * MOE_A2A_OPT_GEMM_TILE forces a form where the shape allows it: 256 the 256 x 256 tiles, 129 the
- * 256 x 128 tiles, 130 those with one partial product per shard, 128 the 128 x 128 tiles, 32 those
- * with one partial product per shard.  All unsplit forms give identical bits.
+ * 256 x 128 tiles (131 / 132: with 192 / 128 of a tile's rows in use, as the library chooses by itself
+ * when that fills the CUs better), 130 those with one partial product per shard, 128 the 128 x 128
+ * tiles, 32 those with one partial product per shard.  All unsplit forms give identical bits.
  */
 size_t gemm_rs_workspace_bytes(int M, int N, int K, int W);
 int gemm_rs_forward(const void* input, const void* weight, const void* bias, void* out, int M, int N, int K, int W,

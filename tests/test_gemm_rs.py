@@ -210,11 +210,12 @@ def test_reference_shapes_at_full_size(gpu_device, spec):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("form", [256, 129, 130, 128, 32])
+@pytest.mark.parametrize("form", [256, 129, 131, 132, 130, 128, 32])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("k", [1024, 1440, 4 * 72], ids=["k256", "k360", "k72"])
 def test_each_kernel_form(gpu_device, options, form, dtype, k):
-    """256 x 256 tiles, 256 x 128 tiles (129; 130: with per-shard partial products), 128 x 128 tiles and
+    """256 x 256 tiles, 256 x 128 tiles (129; 131 / 132: 192 / 128 of their rows in use, the former on
+    the map that deals the tiles out evenly; 130: with per-shard partial products), 128 x 128 tiles and
     their per-shard partial products (32) on one shape with ragged
     edges (M and N not multiples of the tiles); local K a multiple of the 64-column slab, five slabs
     and a short one (360: the wide tiles start the last slab of a shard early and mask what it
@@ -255,7 +256,7 @@ def test_local_k_with_a_short_last_slab_and_one_rank(gpu_device):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("form", [256, 129, 130, 128, 32])
+@pytest.mark.parametrize("form", [256, 129, 131, 130, 128, 32])
 def test_shards_with_gaps_between_them(gpu_device, options, form):
     """Shard strides of the C ABI: the shards of each operand lie further apart than their size."""
     options.set("GEMM_TILE", form)
