@@ -342,7 +342,9 @@ int moe_a2a_expert_gemm_q8(const void* x, const float* x_scale, const void* w_q,
  * than 256 rows, go through moe_a2a_expert_gemm_q8 (any f32 scale).  The option
  * MOE_A2A_OPT_GEMM_TILE = 256 forces the tiles, 32 / 128 the kernels of moe_a2a_expert_gemm_q8,
  * MOE_A2A_OPT_GEMM_STAGED = 1 the register-staged four-wave loop of the tiles, 2 the four-wave loop
- * with slabs sent memory -> LDS (Kd % 256 == 0).  Arguments as for
+ * with slabs sent memory -> LDS (Kd % 256 == 0), 3 / 4 the eight-wave loop with / without the early
+ * requests for the weight rows that segments of less than 192 rows on average get by themselves.
+ * Arguments as for
  * moe_a2a_expert_gemm_q8 with x_scale required.  No counterpart in the reference.
  */
 int moe_a2a_expert_gemm_mx8(const void* x_q, const float* x_scale, const void* w_q, const float* w_scale,
@@ -382,7 +384,9 @@ const char* moe_a2a_kernel_name(int kernel_id);
 #define MOE_A2A_OPT_ROUTE_TILE 0    /* 1: moe_a2a_route_dispatch takes the token-tile kernel at any size   */
 #define MOE_A2A_OPT_GEMM_TILE 1     /* 32 | 128 | 256: tile family of the expert GEMM entry points          */
 #define MOE_A2A_OPT_GEMM_STAGED 2   /* 1: register-staged form of the weight-streaming / scaled-MFMA loops;
-                                       2: four-wave forms of moe_a2a_expert_gemm_mx8 / _q8 with fp8 rows    */
+                                       2: four-wave forms of moe_a2a_expert_gemm_mx8 / _q8 with fp8 rows;
+                                       3 | 4: moe_a2a_expert_gemm_mx8's eight-wave loop with | without early
+                                       requests for the weight rows                                        */
 #define MOE_A2A_OPT_COMBINE_LANES 3 /* lanes of a combine workgroup at cache-resident sizes (64 .. 512)     */
 #define MOE_A2A_OPT_COMBINE_VPL 4   /* 2: two row vectors per lane in the combine at cache-resident sizes   */
 #define MOE_A2A_OPT_TIMER_EVENT_FLAGS 5 /* hipEventCreateWithFlags value for the launch timer's events    */

@@ -216,13 +216,14 @@ def test_expert_gemm_block_quantised_weights(gpu_device, options, E, K, T, H, N,
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("padded", [False, True], ids=["compact", "padded"])
-@pytest.mark.parametrize("form", [0, 2, 1], ids=["eight", "direct", "staged"])
+@pytest.mark.parametrize("form", [4, 3, 2, 1], ids=["eight", "eight-early-b", "direct", "staged"])
 def test_expert_gemm_power_of_two_scales(gpu_device, options, E, K, T, H, N, W, zipf, dtype, padded, form):
     """fp8 rows and fp8 weights whose scales are powers of two, multiplied by the fp8 matrix
     instruction with the scales as its block exponents, against the f32 matmul of the
     dequantised operands; the fp8 x fp8 kernel with the fold on the vector units, which takes
     any f32 scale, has to agree with it to f32 summation order.  All forms of the tiled kernel:
-    eight waves on slabs of 128 columns (hidden sizes from 256), four waves with slabs of 64 columns
+    eight waves on slabs of 128 columns (hidden sizes from 256; with and without the early requests for the
+    rows of the weights that short segments get by themselves), four waves with slabs of 64 columns
     sent memory -> LDS directly (multiples of 256) and staged through registers (every hidden size)."""
     options.set("GEMM_TILE", "256")  # the tiles at every segment length
     options.set("GEMM_STAGED", form)
@@ -245,7 +246,7 @@ def test_expert_gemm_power_of_two_scales(gpu_device, options, E, K, T, H, N, W, 
 
 
 @pytest.mark.parametrize("form", ["16bit-32", "16bit-128", "16bit-256", "q8-32", "q8-32staged", "q8-128", "q8-256",
-                                  "mx-eight", "mx-direct", "mx-staged"])
+                                  "mx-eight", "mx-early", "mx-direct", "mx-staged"])
 def test_padded_overflow_stays_inside_the_buffers(gpu_device, options, form):
     """Padded layout with a LAST expert that receives more rows than max_recv (routing folds the
     surplus onto the segment's last row and raises the overflow bit; counts stay the true numbers):
@@ -265,6 +266,8 @@ def test_padded_overflow_stays_inside_the_buffers(gpu_device, options, form):
         options.set("GEMM_STAGED", 1)
     if tile == "direct":
         options.set("GEMM_STAGED", 2)
+    if tile in ("eight", "early"):  # the eight-wave loop without / with the early requests for the weight rows
+        options.set("GEMM_STAGED", 4 if tile == "eight" else 3)
     fp8 = {"16bit": False, "q8": True, "mx": "pow2"}[kind]
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, W, fp8_dispatch=fp8, padded=True, max_recv=max_recv)
@@ -451,15 +454,20 @@ def walk_cases():
 
 
 @pytest.mark.parametrize("name,counts", walk_cases(), ids=[c[0] for c in walk_cases()])
-@pytest.mark.parametrize("fmt", ["16bit", "mx", "f32scale"])
+@pytest.mark.parametrize("fmt", ["16bit", "16bit-early-b", "mx", "mx-early-b", "f32scale"])
 @pytest.mark.parametrize("N", [256, 640])
 def test_eight_wave_tile_walk_on_odd_segment_tables(gpu_device, options, name, counts, fmt, N):
     """The eight-wave kernels give every expert's m-tiles to one die's workgroups, in groups of at
     most four.  Segment tables that stress that walk: one expert with many tiles, tile-exact and
     one-row segments between runs of empty experts, the largest expert count, rows only at the two
-    ends; one n-tile and a ragged last n-tile; each operand format's eight-wave kernel forced."""
+    ends; one n-tile and a ragged last n-tile; each operand format's eight-wave kernel forced, the two with
+    two slab buffers in both forms (the rows of the weights requested before the slab's last quarter, or
+    early, behind a second barrier, as short segments get them by default)."""
     dtype, H = torch.bfloat16, 256
+    fmt, _, early = fmt.partition("-")
     options.set("GEMM_TILE", "128" if fmt == "f32scale" else "256")
+    if fmt != "f32scale":
+        options.set("GEMM_STAGED", 3 if early else 4)
     cfg, world, weights = make_counts(counts, H, N, dtype, seed=len(counts) + N)
     x, idx, w, rs = concat_world(world, gpu_device)
     fp8 = {"16bit": False, "mx": "pow2", "f32scale": True}[fmt]
