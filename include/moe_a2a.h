@@ -276,9 +276,10 @@ int moe_a2a_forward_launches(int T, int K, int H, int max_recv, int in_type, int
  * this is the grouped matrix product a real MoE layer runs there.
  *   x[rows, Kd], weights[E, N, Kd], y[rows, N]: 16-bit elements of elem_type, f32 accumulation,
  *   Kd % 64 == 0, N % 8 == 0, 16-byte aligned.
- * Three kernels with identical results: 128 x 128 output tiles; 256 x 256 tiles when segments are
- * long (R >= 96 * E and N >= 256); 32 x 128 tiles that stream the weights when segments are short
- * (R <= 32 * E and Kd % 128 == 0).  The option MOE_A2A_OPT_GEMM_TILE = 32, 128 or 256 forces one.
+ * Three kernels with identical results: 256 x 256 tiles (R > 32 * E and N >= 256; for segments of
+ * less than 192 rows on average in a form that requests the weight rows early,
+ * MOE_A2A_OPT_GEMM_STAGED = 3 / 4 forces it on / off); 32 x 128 tiles that stream the weights when
+ * segments are short (R <= 32 * E and Kd % 128 == 0); 128 x 128 output tiles for what is left.  The option MOE_A2A_OPT_GEMM_TILE = 32, 128 or 256 forces one.
  * Padded layout: a segment longer than max_recv (routing raised MOE_A2A_STATUS_OVERFLOW) is
  * multiplied over its first max_recv rows only, so no tile leaves the segment or the buffers.
  */

@@ -70,7 +70,7 @@ def test_expert_gemm_matches_f32_reference(gpu_device, options, E, K, T, H, N, W
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_both_tile_sizes_give_the_same_bits(gpu_device, options, E, K, T, H, N, zipf, dtype):
     """The two kernels accumulate over K in the same order, so their outputs are identical; the
-    default choice for these shapes (R >= 96 E) is the wide one."""
+    default choice for these shapes (R > 32 E) is the wide one."""
     cfg, world, weights = make(E, K, T, H, N, 1, dtype, seed=7 * E + T, zipf=zipf)
     x, idx, w, rs = concat_world(world, gpu_device)
     ata = HipAllToAll(cfg, 0, 1)
